@@ -1,5 +1,5 @@
 """Re-measure the large-M rows of ops/gemm_plan.json with the HB configs of gemm_lg.hip (cfg 88 / 89: the 4-wave
-three-barrier slab loop + LDS-staged epilogue, profiles/r6_gemm_isa_diff.md) among the candidates, and write the
+three-barrier slab loop + LDS-staged epilogue) among the candidates, and write the
 updated plan.
 
 For every plan key (N, K, epilogue) and every M row >= --min-m (plus --add-ms rows for keys whose table stops early):

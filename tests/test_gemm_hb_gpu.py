@@ -1,5 +1,5 @@
-"""The HB configs of gemm_lg.hip (81-90: one wave per SIMD, 128 x 128 outputs per wave, the three-barrier slab loop
-of profiles/r6_gemm_isa_diff.md; 88-90 with the LDS-staged epilogue and split-K) against fp32, in every epilogue mode.
+"""The HB configs of gemm_lg.hip (81-90: one wave per SIMD, 128 x 128 outputs per wave, the three-barrier slab
+loop; 88-90 with the LDS-staged epilogue and split-K) against fp32, in every epilogue mode.
 
 Shapes cover what the production plan never shows at once: M and N that are not tile multiples (partial x tiles,
 partial W tiles in the plain epilogue), K of one slab, an odd number of slabs (the loop is unrolled by two), the
