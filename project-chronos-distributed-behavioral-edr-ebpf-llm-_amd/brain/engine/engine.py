@@ -45,7 +45,8 @@ import numpy as np
 import torch
 
 from ... import ops
-from ...models.llama import KVCache, LlamaModel, StepBatch, build_model, h2d, make_prefill_batch
+from ...models.llama import StepBatch, h2d
+from ...models.registry import build_model
 from ...parallel.tp import TPContext
 from ...utils import trace
 from ..constrain import DONE, GrammarBank
@@ -58,8 +59,9 @@ _PHASE_SYNC = os.environ.get("CHRONOS_PHASE_SYNC", "0") not in ("", "0")
 
 @dataclass
 class EngineConfig:
-    model: str = "llama3-8b"
+    model: str = "llama3-8b"       # a preset name of any registered family, or a checkpoint directory
     checkpoint: Optional[str] = None
+    dtype: str = "bf16"            # activation / weight dtype: "bf16", or "fp32" for the families that run in it
     tokenizer: Optional[str] = None
     device: str = "cuda"
     seed: int = 0
@@ -216,7 +218,7 @@ class _Snapshot:
 
 
 class Engine:
-    def __init__(self, cfg: EngineConfig, tp: TPContext | None = None, model: LlamaModel | None = None,
+    def __init__(self, cfg: EngineConfig, tp: TPContext | None = None, model=None,
                  tokenizer=None, cp: TPContext | None = None):
         """``cp``: a context-parallel group (full weights on every rank, parallel/context_parallel.py).  Its ranks
         run this engine in lockstep (same submissions, same order); long prefill chunks are split across them and
@@ -236,11 +238,14 @@ class Engine:
             torch.cuda.set_device(self.device)
             ops.load()  # the HIP library must load on a GPU engine — never a silent eager fallback
             ops.device_init()
-        self.tok = tokenizer or load_tokenizer(cfg.tokenizer)
         t0 = time.perf_counter()
         self.model = model or build_model(cfg.model, self.device, self.tp, cfg.seed, cfg.checkpoint,
-                                          max_position=cfg.max_model_len + 16, weight_dtype=cfg.weight_dtype)
+                                          max_position=cfg.max_model_len + 16, weight_dtype=cfg.weight_dtype,
+                                          dtype=cfg.dtype)
         self.load_seconds = time.perf_counter() - t0
+        # a model whose vocabulary is not the Llama-3 one and that ships no tokenizer.json gets the byte tokenizer
+        self.tok = tokenizer or load_tokenizer(cfg.tokenizer or cfg.checkpoint or cfg.model,
+                                               vocab_size=self.model.cfg.vocab_size)
         self.model.sequence_parallel = cfg.tp_sequence_parallel and self.tp.world > 1
         self.model.decode_overlap_rows = cfg.tp_decode_overlap if self.tp.world > 1 else 0
         mc = self.model.cfg
@@ -262,7 +267,7 @@ class Engine:
             if self.device.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(self.device)
                 budget = max(0.0, free * cfg.kv_fraction - cfg.reserve_gb * 2**30)
-                nb = int(budget // KVCache.bytes_per_block(mc, self.tp, bs, cfg.kv_dtype))
+                nb = int(budget // self.model.cache_bytes_per_block(bs, cfg.kv_dtype))
                 nb = max(2, min(nb, need))
             else:
                 nb = need
@@ -273,11 +278,13 @@ class Engine:
                 t = torch.tensor([nb], dtype=torch.int64, device=self.device)
                 dist.all_reduce(t, op=dist.ReduceOp.MIN, group=grp.group)
                 nb = int(t.item())
-        self.kv = KVCache(mc, self.tp, nb, bs, self.device, cfg.kv_dtype, cfg.kv_scale, cfg.kv_scale)
+        self.kv = self.model.make_cache(nb, bs, cfg.max_slots, cfg.kv_dtype, cfg.kv_scale, cfg.kv_scale)
+        # sequences with recurrent state cannot adopt another sequence's pages: the state after a prefix is not cached
+        self._prefix_cache = cfg.prefix_cache and not self.model.recurrent
         if cfg.kv_alloc not in ("auto", "lazy", "full"):
             raise ValueError(f"kv_alloc must be auto, lazy or full, not {cfg.kv_alloc!r}")
         self.kv_alloc = cfg.kv_alloc if cfg.kv_alloc != "auto" else ("full" if nb >= need else "lazy")
-        self.blocks = BlockManager(nb, bs, prefix_cache=cfg.prefix_cache, partial_prefix=cfg.partial_prefix)
+        self.blocks = BlockManager(nb, bs, prefix_cache=self._prefix_cache, partial_prefix=cfg.partial_prefix)
         # ---- slot state (device) ----
         S, dev = cfg.max_slots, self.device
         i32 = dict(dtype=torch.int32, device=dev)
@@ -294,6 +301,9 @@ class Engine:
         self.s_out = torch.zeros(S, cfg.max_out, **i32)
         self.s_bt = torch.zeros(S, self.max_blocks_per_seq, **i32)
         self.s_row = torch.full((S,), -1, **i32)
+        # state slot of each decode row: its own index while a sequence runs in it, else the cache's scratch row (a
+        # decode step covers every row of its bucket, also rows whose prompt is still prefilling)
+        self.s_slot = torch.full((S,), S, **i32)
         self.ar = torch.arange(S + 1, **i32)
         self.ar64 = torch.arange(S, dtype=torch.int64, device=dev)
         # ---- scheduling state ----
@@ -323,7 +333,8 @@ class Engine:
         # cascade prefix state: device [P, block ids...] read by the decode graph, its O / lse scratch, host copy
         self._casc = None
         self._casc_cur: tuple = ()
-        if self.device.type == "cuda" and cfg.cascade and self.model.hq % self.model.hkv == 0 and \
+        if self.device.type == "cuda" and cfg.cascade and not self.model.recurrent and \
+                self.model.hq % self.model.hkv == 0 and \
                 16 % (self.model.hq // self.model.hkv) == 0:
             self._casc = (torch.zeros(1 + cfg.cascade_max_blocks, dtype=torch.int32, device=dev),
                           torch.empty(S, self.model.hq, 128, dtype=torch.bfloat16, device=dev),
@@ -483,6 +494,7 @@ class Engine:
             self.s_bt.index_fill_(0, idx, 0)
             self.s_pos.index_fill_(0, idx, 0)
             self.s_ctx.index_fill_(0, idx, 1)
+            self.s_slot.index_fill_(0, idx, self.cfg.max_slots)
         return out
 
     def fail_all(self, error: str) -> list[Request]:
@@ -504,7 +516,7 @@ class Engine:
         S = self.cfg.max_slots
         self.free_slots = list(range(S - 1, -1, -1))
         self.blocks = BlockManager(self.blocks.num_blocks, self.blocks.block_size,
-                                   prefix_cache=self.blocks.prefix_cache, partial_prefix=self.cfg.partial_prefix)
+                                   prefix_cache=self._prefix_cache, partial_prefix=self.cfg.partial_prefix)
         self._casc_cur = ()
         try:
             if self._casc is not None:
@@ -513,6 +525,7 @@ class Engine:
             self.s_bt.zero_()
             self.s_pos.zero_()
             self.s_ctx.fill_(1)
+            self.s_slot.fill_(S)
         except Exception:  # noqa: BLE001 — a dead device must not stop the error replies below
             log.exception("slot state reset after a failed step")
         out = []
@@ -737,6 +750,7 @@ class Engine:
         self.s_bt.index_fill_(0, idx, 0)
         self.s_pos.index_fill_(0, idx, 0)
         self.s_ctx.index_fill_(0, idx, 1)
+        self.s_slot.index_fill_(0, idx, self.cfg.max_slots)
 
     def _grow_for(self, k: int) -> None:
         """Lazy KV: every running row may write k more KV positions in the launch about to be queued (a decode burst
@@ -808,6 +822,7 @@ class Engine:
         self.s_rem[sl] = dv(torch.tensor([r.num_predict for r in done_reqs], dtype=torch.int32))
         self.s_pos[sl] = dv(plen - 1)
         self.s_ctx[sl] = dv(plen)
+        self.s_slot[sl] = dv(slots.to(torch.int32))
         self.s_nout.index_fill_(0, sl, 0)
         self.s_temp[sl] = dv(torch.tensor([r.temperature for r in done_reqs], dtype=torch.float32))
         self.s_seed[sl] = dv(torch.tensor([r.seed for r in done_reqs], dtype=torch.int32))
@@ -849,8 +864,8 @@ class Engine:
             chunks, starts, bts, reqs = self._fit(chunks, starts, bts, reqs)
             ntok = sum(len(c) for c in chunks)
             split = 2 if (self.tp.world > 1 and self.cfg.tp_overlap and ntok >= self.cfg.tp_overlap_min_tokens) else 1
-            sb = make_prefill_batch(chunks, starts, bts, self.model.cfg, self.tp, self.device,
-                                    max_blocks=self.max_blocks_per_seq, nqt=self.cfg.prefill_nqt, split=split)
+            sb = self.model.prefill_batch(chunks, starts, bts, [r.slot for r in reqs],
+                                          max_blocks=self.max_blocks_per_seq, nqt=self.cfg.prefill_nqt, split=split)
             logits = self.model.forward(sb, self.kv)
         done_rows, done_reqs = self._prefill_done(reqs, chunks)
         if not done_reqs:
@@ -887,12 +902,13 @@ class Engine:
         budget = min(self._ramp, max(self.cfg.mixed_prefill_tokens, self.cfg.mixed_ratio * n))
         self._ramp = min(4 * self._ramp, self._chunk)
         chunks, starts, bts, reqs = self._fit(*self._gather_prefill(budget))
-        sb = make_prefill_batch(chunks, starts, bts, self.model.cfg, self.tp, self.device,
-                                max_blocks=self.max_blocks_per_seq, nqt=self.cfg.prefill_nqt)
+        sb = self.model.prefill_batch(chunks, starts, bts, [r.slot for r in reqs],
+                                      max_blocks=self.max_blocks_per_seq, nqt=self.cfg.prefill_nqt)
         tp_, bp = sum(len(c) for c in chunks), len(chunks)
         self._update_casc()
         sb.dec = StepBatch(self.s_ids[:n], self.s_pos[:n], self.ar[:n], self.s_bt[:n], self.ar[:n + 1], self.s_ctx[:n],
-                           self.ar64[:n], None, n, 1, self._nsplit(n, self._ctx_class()), casc=self._casc)
+                           self.ar64[:n], None, n, 1, self._nsplit(n, self._ctx_class()), casc=self._casc,
+                           slots=self.s_slot[:n], max_q=1)
         sb.last_idx = torch.cat([sb.last_idx, tp_ + self.ar64[:n]])
         logits = self.model.forward(sb, self.kv)
         done_rows, done_reqs = self._prefill_done(reqs, chunks)
@@ -931,7 +947,7 @@ class Engine:
 
     def _decode_once(self, n: int, nsplit: int) -> None:
         sb = StepBatch(self.s_ids[:n], self.s_pos[:n], self.ar[:n], self.s_bt[:n], self.ar[:n + 1], self.s_ctx[:n],
-                       self.ar64[:n], None, n, 1, nsplit, casc=self._casc)
+                       self.ar64[:n], None, n, 1, nsplit, casc=self._casc, slots=self.s_slot[:n], max_q=1)
         logits = self.model.forward(sb, self.kv)
         ops.constrained_sample(logits, None, self.bank.next, self.bank.dist, DONE, self.s_state[:n], self.s_rem[:n],
                                self.s_temp[:n], self.s_seed[:n], self.s_ids[:n], self.s_pos[:n], self.s_ctx[:n],
@@ -1116,6 +1132,7 @@ class Engine:
         self.s_bt.index_fill_(0, idx, 0)
         self.s_pos.index_fill_(0, idx, 0)
         self.s_ctx.index_fill_(0, idx, 1)
+        self.s_slot.index_fill_(0, idx, self.cfg.max_slots)
         self.stats["completed"] += len(done)
         self.stats["generated_tokens"] += sum(len(r.out_ids) for r in done)
         self._compact()
@@ -1183,8 +1200,8 @@ class Engine:
         # The flash prefill kernel (nqt=8) runs one workgroup per (tile, kv head) over the whole context: at 128k
         # that is 8 workgroups streaming 16 GiB of KV per jump (14 ms/token decode instead of 6-7).
         nqt = 2 if max(pos0) > 4096 else self.cfg.prefill_nqt
-        sb = make_prefill_batch([ids[n0 - 1:] for _, ids, _, n0, _ in rows], pos0, [r.blocks for r, *_ in rows],
-                                self.model.cfg, self.tp, self.device, max_blocks=self.max_blocks_per_seq, nqt=nqt)
+        sb = self.model.prefill_batch([ids[n0 - 1:] for _, ids, _, n0, _ in rows], pos0, [r.blocks for r, *_ in rows],
+                                      [r.slot for r, *_ in rows], max_blocks=self.max_blocks_per_seq, nqt=nqt)
         logits = self.model.forward(sb, self.kv)
         i32 = lambda x: dv(torch.tensor(x, dtype=torch.int32))  # noqa: E731
         sl = dv(torch.tensor([r.slot for r, *_ in rows], dtype=torch.int64))
@@ -1225,10 +1242,14 @@ class Engine:
         for t in (self.s_ids, self.s_pos, self.s_ctx, self.s_state, self.s_rem, self.s_nout, self.s_seed, self.s_temp,
                   self.s_topk, self.s_topp, self.s_out, self.s_bt):
             t[di] = t[si]
+        if self.model.recurrent:  # the sequences' recurrent state follows them
+            self.kv.move_slots(si, di)
+        self.s_slot[di] = di.to(torch.int32)
         self.s_state.index_fill_(0, si, -1)
         self.s_bt.index_fill_(0, si, 0)
         self.s_pos.index_fill_(0, si, 0)
         self.s_ctx.index_fill_(0, si, 1)
+        self.s_slot.index_fill_(0, si, self.cfg.max_slots)
         moved = {}
         for s, d in zip(movers, dst):
             r = self.running.pop(s)

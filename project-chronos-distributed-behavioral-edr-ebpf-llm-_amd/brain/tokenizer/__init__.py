@@ -175,9 +175,37 @@ class HFTokenizer(_Base):
         return self._bytes
 
 
-def load_tokenizer(path: str | None = None) -> _Base:
+class ByteTokenizer(_Base):
+    """Tokenizer of last resort for a model whose vocabulary is not the Llama-3 one and that ships no tokenizer
+    file: token i < 256 is byte i, the two highest ids are <bos> and <eot>, every other id decodes to nothing.  A
+    vocabulary of fewer than 258 entries keeps its low bytes only."""
+
+    def __init__(self, vocab_size: int):
+        if vocab_size < 4:
+            raise ValueError("the byte tokenizer needs at least 4 token ids")
+        self.vocab_size = vocab_size
+        self.bos_id, self.eot_id = vocab_size - 2, vocab_size - 1
+        self.stop_ids = (self.eot_id,)
+        self.n_bytes = min(256, vocab_size - 2)
+        self._bytes = [bytes([i]) if i < self.n_bytes else b"" for i in range(vocab_size)]
+
+    def encode(self, text: str) -> list[int]:
+        return [b for b in text.encode("utf-8") if b < self.n_bytes]
+
+    def token_bytes_list(self) -> list[bytes]:
+        return self._bytes
+
+    def chat_ids(self, prompt: str, system: str | None = None, raw: bool = False) -> list[int]:
+        return [self.bos_id] + self.encode((system + "\n" if system and not raw else "") + prompt)
+
+
+def load_tokenizer(path: str | None = None, vocab_size: int | None = None) -> _Base:
+    """``path``: a tokenizer.json or a directory that may hold one.  ``vocab_size``: the model's; anything but the
+    Llama-3 size without a tokenizer file gets the :class:`ByteTokenizer`."""
     if path:
         cand = os.path.join(path, "tokenizer.json") if os.path.isdir(path) else path
-        if os.path.exists(cand):
+        if os.path.isfile(cand) and cand.endswith(".json"):
             return HFTokenizer(cand)
+    if vocab_size is not None and vocab_size != VOCAB_SIZE:
+        return ByteTokenizer(vocab_size)
     return ChronosBPE()

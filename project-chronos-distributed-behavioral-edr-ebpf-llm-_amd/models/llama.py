@@ -495,6 +495,10 @@ class StepBatch:
     # the split-K decode kernel with all of a sequence's tokens in one pass over its K/V (ops.paged_attention
     # max_q) instead of the prefill tiles, whose per-tile workgroups each stream the whole context
     rows_dec: Optional[tuple] = None
+    # models with per-sequence recurrent state (models/hybrid.py): the state slot of every sequence, [B] int32, and
+    # the most tokens any sequence brings in this step (a launch-shape hint)
+    slots: Optional[torch.Tensor] = None
+    max_q: int = 0
 
 
 # decode-form attention for tiny chunks over long contexts (StepBatch.rows_dec): at least this much context (the
@@ -504,7 +508,7 @@ ROWS_DEC_MIN_CTX = int(os.environ.get("CHRONOS_ROWS_DEC_MIN_CTX", "2048"))
 
 def make_prefill_batch(prompts: list[list[int]], starts: list[int], block_tables: list[list[int]], cfg: LlamaConfig,
                        tp: TPContext, device, max_blocks: int | None = None, nqt: int = 2,
-                       ctx_totals: list[int] | None = None, split: int = 1) -> StepBatch:
+                       ctx_totals: list[int] | None = None, split: int = 1, slots: list[int] | None = None) -> StepBatch:
     """Host builder for a (chunked) prefill step.  prompts[b] are the tokens of this chunk, starts[b] the position of
     its first token (prefix already in the cache).  ``split > 1`` also builds that many token-balanced micro-batches
     of whole sequences (``StepBatch.parts``) for communication/compute overlap under tensor parallelism."""
@@ -543,6 +547,9 @@ def make_prefill_batch(prompts: list[list[int]], starts: list[int], block_tables
     mq = max((len(t) for t in prompts), default=0)
     if prompts and mq * (hq // hkv) <= 16 and max(ctx) >= ROWS_DEC_MIN_CTX and ctx_totals is None:
         sb.rows_dec = (mq, ops.pick_nsplit(len(prompts) * hkv, max(ctx)))
+    sb.max_q = mq
+    if slots is not None:
+        sb.slots = it(list(slots))
     return to_device(sb, device)
 
 
@@ -560,7 +567,7 @@ def to_device(sb: StepBatch, device) -> StepBatch:
     mv = lambda t: h2d(t, device)  # noqa: E731
     return StepBatch(mv(sb.ids), mv(sb.pos), mv(sb.tok_seq), mv(sb.block_table), mv(sb.q_start), mv(sb.ctx_len),
                      mv(sb.last_idx), mv(sb.tiles), sb.ntiles, sb.nqt, sb.nsplit, sb.parts, sb.cp, sb.dec, sb.casc,
-                     sb.rows_dec)
+                     sb.rows_dec, mv(sb.slots), sb.max_q)
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -584,6 +591,24 @@ class LlamaModel:
         # HIP stream, each overlapping the other half's attention / MLP (0 = off)
         self.decode_overlap_rows = 0
         self._comm = None
+
+    # ---- what the engine asks of any model it serves (models/registry.py) -------------------------------------------
+    recurrent = False  # no per-sequence state beyond the paged KV: prefixes can be shared between sequences
+
+    def make_cache(self, num_blocks: int, block_size: int, slots: int, kv_dtype: str = "bf16", k_scale: float = 1.0,
+                   v_scale: float = 1.0) -> "KVCache":
+        return KVCache(self.cfg, self.tp, num_blocks, block_size, self.device, kv_dtype, k_scale, v_scale)
+
+    def cache_bytes_per_block(self, block_size: int, kv_dtype: str = "bf16") -> int:
+        return KVCache.bytes_per_block(self.cfg, self.tp, block_size, kv_dtype)
+
+    def prefill_batch(self, chunks, starts, block_tables, slots=None, max_blocks=None, nqt: int = 2, split: int = 1,
+                      want=None) -> "StepBatch":
+        sb = make_prefill_batch(chunks, starts, block_tables, self.cfg, self.tp, self.device, max_blocks=max_blocks,
+                                nqt=nqt, split=split)
+        if want is not None:
+            sb.last_idx = h2d(torch.tensor(list(want), dtype=torch.int64), self.device)
+        return sb
 
     # ---- one micro-batch's pieces of a layer (bf16: x is a tensor; W8A8: x is (e4m3 bytes, row scales)) ----------
     def _norm(self, h, st: dict, w: torch.Tensor, first: bool = False, reduce: bool = False):

@@ -1,0 +1,119 @@
+"""Ops of the hybrid decoders (recurrent matrix-memory layers, latent attention, mixtures of experts, layer norms on
+a float32 residual stream): gfx950 HIP kernels on the GPU (csrc/kernels/hybrid_*.hip), the PyTorch references of
+:mod:`.hybrid_ref` on the CPU.
+
+As everywhere in :mod:`chronos.ops` a GPU tensor never falls back silently: it goes to ``torch.ops.chronos.hy_*`` or
+raises.  ``CHRONOS_HYBRID_REF=1`` is a bring-up switch that runs the PyTorch references on GPU tensors (it syncs with
+the host and cannot be captured into a graph).
+
+Activations are bfloat16 or float32 (one build serves both: the kernels are instantiated for the two); the residual
+stream, norms, recurrent state, gates, router and attention scores are float32 in either mode.
+"""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from . import hybrid_ref as ref
+from .hybrid_ref import ACT_GELU, ACT_RELU2  # noqa: F401
+
+_REF_ON_GPU = os.environ.get("CHRONOS_HYBRID_REF", "0") not in ("", "0")
+
+
+def _gpu(t: torch.Tensor) -> bool:
+    return t.is_cuda and not _REF_ON_GPU
+
+
+def _k():
+    from . import _k as k
+
+    return k()
+
+
+def _f32(act_dtype) -> bool:
+    return act_dtype == torch.float32
+
+
+def matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x @ w.T: the framework's routed projection GEMMs for bfloat16, the library's float32 GEMM otherwise."""
+    if x.dtype == torch.bfloat16:
+        from . import linear
+
+        return linear(x, w)
+    return torch.matmul(x, w.t())
+
+
+def embed_rows(ids, table, act_dtype):
+    """(float32 residual rows, the same rows in the activation dtype)."""
+    if _gpu(table):
+        x = _k().hy_embed(ids, table)
+        return x, (x if _f32(act_dtype) else _k().hy_cast_bf16(x))
+    return ref.embed_rows(ids, table, act_dtype)
+
+
+def layer_norm(x, w, eps: float, act_dtype):
+    if _gpu(x):
+        return _k().hy_layer_norm(x, w, eps, _f32(act_dtype))
+    return ref.layer_norm(x, w, eps, act_dtype)
+
+
+def add_layer_norm(y, x, w, eps: float, act_dtype):
+    """x (float32 residual, in place) <- x + layer_norm(y) * w; returns the updated rows in the activation dtype
+    (x itself when that is float32)."""
+    if _gpu(x):
+        h = _k().hy_add_layer_norm(y, x, w, eps, _f32(act_dtype))
+        return x if _f32(act_dtype) else h
+    return ref.add_layer_norm(y, x, w, eps, act_dtype)
+
+
+def rowdot(h, w, bias=None):
+    if _gpu(h):
+        return _k().hy_rowdot(h, w, bias)
+    return ref.rowdot(h, w, bias)
+
+
+def act_inplace(x, kind: int):
+    if _gpu(x):
+        _k().hy_act(x, kind)
+        return x
+    return ref.act_inplace(x, kind)
+
+
+def mlstm_scan(proj, gate_pre, q_start, pos0, slots, S, n, m, H: int, D: int, Dv: int, cap: float, max_q: int = 0):
+    """``max_q``: the most tokens any sequence brings in this step (a launch-shape hint; 0 = unknown)."""
+    if _gpu(proj):
+        return _k().hy_mlstm_scan(proj, gate_pre, q_start, pos0, slots, S, n, m, H, D, Dv, cap)
+    return ref.mlstm_scan(proj, gate_pre, q_start, pos0, slots, S, n, m, H, D, Dv, cap)
+
+
+def mlstm_out(o, proj, g_off: int, norm_w, eps: float, act_dtype):
+    if _gpu(o):
+        return _k().hy_mlstm_out(o, proj, g_off, norm_w, eps, _f32(act_dtype))
+    return ref.mlstm_out(o, proj, g_off, norm_w, eps, act_dtype)
+
+
+def latent_prep(q, dkv, pos, tok_seq, block_table, w_norm, eps: float, cos_sin, dims: int, rank: int, cache) -> None:
+    if _gpu(q):
+        _k().hy_latent_prep(q, dkv, pos, tok_seq, block_table, w_norm, eps, cos_sin, dims, rank, cache)
+    else:
+        ref.latent_prep(q, dkv, pos, tok_seq, block_table, w_norm, eps, cos_sin, dims, rank, cache)
+
+
+def latent_attention(qa, cache, block_table, q_start, pos, gate, scale: float, rank: int, act_dtype, max_q: int):
+    """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid)."""
+    if _gpu(qa):
+        return _k().hy_latent_attention(qa, cache, block_table, q_start, pos, gate, scale, rank, max_q)
+    return ref.latent_attention(qa, cache, block_table, q_start, pos, gate, scale, rank, act_dtype)
+
+
+def moe_route(h, w_router, correction, top: int):
+    if _gpu(h):
+        return _k().hy_moe_route(h, w_router, correction, top)
+    return ref.moe_route(h, w_router, correction, top)
+
+
+def moe_ffn(h, idx, wt, w_up, w_down, act: int, act_dtype):
+    if _gpu(h):
+        return _k().hy_moe_ffn(h, idx, wt, w_up, w_down, act)
+    return ref.moe_ffn(h, idx, wt, w_up, w_down, act, act_dtype)
