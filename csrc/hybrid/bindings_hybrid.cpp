@@ -1,0 +1,261 @@
+// bindings_hybrid.cpp — registers the hybrid-decoder kernels (csrc/hybrid/*.hip) as torch.ops.chronos.hy_*.
+//
+// A library of its own (_H), so a model of this family compiles and loads only these kernels.  As in
+// csrc/kernels/bindings.cpp every op checks dtypes, shapes and contiguity on the host before launching and launches on
+// the current HIP stream (graph-capturable; outputs come from torch's caching allocator).
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <tuple>
+
+namespace chronos {
+void launch_hy_embed(const int32_t*, const void*, float*, int, int, bool, hipStream_t);
+void launch_hy_cast_bf16(const float*, uint16_t*, int64_t, hipStream_t);
+void launch_hy_layer_norm(const void*, bool, float*, const float*, void*, bool, int, int, float, hipStream_t);
+void launch_hy_rowdot(const void*, const void*, const float*, float*, int, int, int, bool, hipStream_t);
+void launch_hy_act(void*, int64_t, int, bool, hipStream_t);
+void launch_hy_mlstm_scan(const void*, int, const float*, const int32_t*, const int32_t*, const int32_t*, float*, float*,
+                          float*, float*, float*, float*, float*, int, int, int, int, float, bool, hipStream_t);
+void launch_hy_mlstm_out(const float*, const void*, int, int, const float*, void*, int, int, int, float, bool,
+                         hipStream_t);
+void launch_hy_latent_prep(void*, const void*, const int32_t*, const int32_t*, const int32_t*, int, const float*, float,
+                           const float*, int, int, int, int, int, void*, int, int, bool, hipStream_t);
+bool launch_hy_latent_attention(const void*, const void*, const int32_t*, int, const int32_t*, const int32_t*,
+                                const float*, void*, int, int, int, int, int, int, float, bool, hipStream_t);
+void launch_hy_moe_route(const void*, const void*, const float*, int32_t*, float*, int, int, int, int, bool,
+                         hipStream_t);
+void launch_hy_moe_ffn_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
+                             int, int, int, bool, hipStream_t);
+}  // namespace chronos
+
+namespace {
+
+using at::Tensor;
+
+hipStream_t stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+void need(bool ok, const char* what) { TORCH_CHECK(ok, "chronos hybrid op: ", what); }
+
+bool is_act(const Tensor& t) { return t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat; }
+bool f32(const Tensor& t) { return t.scalar_type() == at::kFloat; }
+void same_act(const Tensor& a, const Tensor& b, const char* what) {
+    need(is_act(a) && a.scalar_type() == b.scalar_type(), what);
+}
+void i32(const Tensor& t, const char* what) { need(t.scalar_type() == at::kInt && t.is_contiguous() && t.is_cuda(), what); }
+void flt(const Tensor& t, const char* what) { need(t.scalar_type() == at::kFloat && t.is_contiguous() && t.is_cuda(), what); }
+
+Tensor hy_embed(const Tensor& ids, const Tensor& table) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(table.device());
+    i32(ids, "embed: ids must be contiguous int32");
+    need(is_act(table) && table.dim() == 2 && table.is_contiguous(), "embed: table [V, d] bf16 or f32");
+    auto x = at::empty({ids.numel(), table.size(1)}, table.options().dtype(at::kFloat));
+    chronos::launch_hy_embed(ids.data_ptr<int32_t>(), table.data_ptr(), x.data_ptr<float>(), (int)ids.numel(),
+                             (int)table.size(1), f32(table), stream());
+    return x;
+}
+
+Tensor hy_cast_bf16(const Tensor& x) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "cast: float32 contiguous input");
+    auto y = at::empty_like(x, x.options().dtype(at::kBFloat16));
+    chronos::launch_hy_cast_bf16(x.data_ptr<float>(), (uint16_t*)y.data_ptr(), x.numel(), stream());
+    return y;
+}
+
+Tensor hy_layer_norm(const Tensor& x, const Tensor& w, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "layer_norm: float32 rows");
+    flt(w, "layer_norm: float32 weight");
+    need(x.dim() == 2 && w.numel() == x.size(1), "layer_norm: weight size");
+    auto h = at::empty_like(x, x.options().dtype(out_f32 ? at::kFloat : at::kBFloat16));
+    chronos::launch_hy_layer_norm(x.data_ptr(), true, nullptr, w.data_ptr<float>(), h.data_ptr(), out_f32,
+                                  (int)x.size(0), (int)x.size(1), (float)eps, stream());
+    return h;
+}
+
+Tensor hy_add_layer_norm(const Tensor& y, Tensor& x, const Tensor& w, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "add_layer_norm: float32 residual");
+    flt(w, "add_layer_norm: float32 weight");
+    need(is_act(y) && y.is_contiguous() && y.dim() == 2 && y.sizes() == x.sizes(), "add_layer_norm: y shape");
+    need(f32(y) == out_f32, "add_layer_norm: y must be in the activation dtype");
+    need(w.numel() == x.size(1), "add_layer_norm: weight size");
+    Tensor h = out_f32 ? at::empty({0}, x.options()) : at::empty_like(x, x.options().dtype(at::kBFloat16));
+    chronos::launch_hy_layer_norm(y.data_ptr(), out_f32, x.data_ptr<float>(), w.data_ptr<float>(),
+                                  out_f32 ? nullptr : h.data_ptr(), out_f32, (int)x.size(0), (int)x.size(1), (float)eps,
+                                  stream());
+    return h;
+}
+
+Tensor hy_rowdot(const Tensor& h, const Tensor& w, const c10::optional<Tensor>& bias) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w, "rowdot: h and w in one activation dtype");
+    need(h.dim() == 2 && w.dim() == 2 && h.is_contiguous() && w.is_contiguous() && h.size(1) == w.size(1), "rowdot: shapes");
+    if (bias) { flt(*bias, "rowdot: float32 bias"); need(bias->numel() == w.size(0), "rowdot: bias size"); }
+    auto out = at::empty({h.size(0), w.size(0)}, h.options().dtype(at::kFloat));
+    chronos::launch_hy_rowdot(h.data_ptr(), w.data_ptr(), bias ? bias->data_ptr<float>() : nullptr, out.data_ptr<float>(),
+                              (int)h.size(0), (int)h.size(1), (int)w.size(0), f32(h), stream());
+    return out;
+}
+
+void hy_act(Tensor& x, int64_t kind) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    need(is_act(x) && x.is_contiguous() && (kind == 0 || kind == 1), "act: contiguous activation tensor, kind 0/1");
+    chronos::launch_hy_act(x.data_ptr(), x.numel(), (int)kind, f32(x), stream());
+}
+
+Tensor hy_mlstm_scan(const Tensor& proj, const Tensor& gate_pre, const Tensor& q_start, const Tensor& pos0,
+                     const Tensor& slots, Tensor& S, Tensor& n, Tensor& m, int64_t H, int64_t D, int64_t Dv, double cap) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+    need(is_act(proj) && proj.dim() == 2 && proj.is_contiguous(), "mlstm_scan: proj [T, C]");
+    need(proj.size(1) >= 2 * H * D + H * Dv, "mlstm_scan: proj narrower than q | k | v");
+    flt(gate_pre, "mlstm_scan: float32 gate pre-activations");
+    const int64_t T = proj.size(0);
+    need(gate_pre.dim() == 2 && gate_pre.size(0) == T && gate_pre.size(1) == 2 * H, "mlstm_scan: gate_pre [T, 2H]");
+    i32(q_start, "mlstm_scan: q_start"); i32(pos0, "mlstm_scan: pos0"); i32(slots, "mlstm_scan: slots");
+    const int64_t B = slots.numel();
+    need(q_start.numel() == B + 1 && pos0.numel() == B, "mlstm_scan: q_start [B+1], pos0 [B], slots [B]");
+    flt(S, "mlstm_scan: S"); flt(n, "mlstm_scan: n"); flt(m, "mlstm_scan: m");
+    need(S.dim() == 4 && S.size(1) == H && S.size(2) == D && S.size(3) == Dv, "mlstm_scan: S [NS, H, D, Dv]");
+    need(n.dim() == 3 && n.size(0) == S.size(0) && n.size(1) == H && n.size(2) == D, "mlstm_scan: n [NS, H, D]");
+    need(m.dim() == 2 && m.size(0) == S.size(0) && m.size(1) == H, "mlstm_scan: m [NS, H]");
+    need(D >= 1 && D <= 512 && H >= 1 && Dv >= 1, "mlstm_scan: 1 <= D <= 512");
+    auto o = at::empty({T, H, Dv}, proj.options().dtype(at::kFloat));
+    auto scratch = at::empty({3, T, H}, proj.options().dtype(at::kFloat));
+    float* sp = scratch.data_ptr<float>();
+    chronos::launch_hy_mlstm_scan(proj.data_ptr(), (int)proj.size(1), gate_pre.data_ptr<float>(),
+                                  q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(), slots.data_ptr<int32_t>(),
+                                  S.data_ptr<float>(), n.data_ptr<float>(), m.data_ptr<float>(), sp, sp + T * H,
+                                  sp + 2 * T * H, o.data_ptr<float>(), (int)B, (int)H, (int)D, (int)Dv, (float)cap,
+                                  f32(proj), stream());
+    return o;
+}
+
+Tensor hy_mlstm_out(const Tensor& o, const Tensor& proj, int64_t g_off, const Tensor& w, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+    flt(o, "mlstm_out: float32 read-out");
+    flt(w, "mlstm_out: float32 weight");
+    need(o.dim() == 3 && is_act(proj) && proj.dim() == 2 && proj.is_contiguous() && proj.size(0) == o.size(0), "mlstm_out: shapes");
+    const int64_t T = o.size(0), H = o.size(1), Dv = o.size(2);
+    need(f32(proj) == out_f32 && g_off >= 0 && g_off + H * Dv <= proj.size(1) && w.numel() == H * Dv, "mlstm_out: gate columns / weight");
+    auto y = at::empty({T, H * Dv}, proj.options());
+    chronos::launch_hy_mlstm_out(o.data_ptr<float>(), proj.data_ptr(), (int)proj.size(1), (int)g_off, w.data_ptr<float>(),
+                                 y.data_ptr(), (int)T, (int)H, (int)Dv, (float)eps, out_f32, stream());
+    return y;
+}
+
+void hy_latent_prep(Tensor& q, const Tensor& dkv, const Tensor& pos, const Tensor& tok_seq, const Tensor& block_table,
+                    const Tensor& w_norm, double eps, const Tensor& cos_sin, int64_t dims, int64_t rank, Tensor& cache) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
+    same_act(q, dkv, "latent_prep: q and dkv in one activation dtype");
+    same_act(q, cache, "latent_prep: the cache holds the activation dtype");
+    need(q.dim() == 3 && q.is_contiguous() && dkv.dim() == 2 && dkv.is_contiguous() && cache.dim() == 3 && cache.is_contiguous(), "latent_prep: layouts");
+    const int64_t T = q.size(0), H = q.size(1), DK = dkv.size(1), R = DK - rank, D = q.size(2) - R;
+    need(dkv.size(0) == T && rank >= 1 && R >= 0 && D >= 0 && cache.size(2) == DK, "latent_prep: sizes");
+    need(dims % 2 == 0 && dims <= R, "latent_prep: rotated columns");
+    i32(pos, "latent_prep: pos"); i32(tok_seq, "latent_prep: tok_seq"); i32(block_table, "latent_prep: block_table");
+    need(pos.numel() == T && tok_seq.numel() == T && block_table.dim() == 2, "latent_prep: per-token metadata");
+    flt(w_norm, "latent_prep: float32 norm weight"); flt(cos_sin, "latent_prep: float32 cos/sin table");
+    need(w_norm.numel() == rank && cos_sin.dim() == 2 && cos_sin.size(1) == dims, "latent_prep: norm weight / table width");
+    chronos::launch_hy_latent_prep(q.data_ptr(), dkv.data_ptr(), pos.data_ptr<int32_t>(), tok_seq.data_ptr<int32_t>(),
+                                   block_table.data_ptr<int32_t>(), (int)block_table.size(1), w_norm.data_ptr<float>(),
+                                   (float)eps, cos_sin.data_ptr<float>(), (int)dims, (int)rank, (int)R, (int)H, (int)D,
+                                   cache.data_ptr(), (int)cache.size(1), (int)T, f32(q), stream());
+}
+
+Tensor hy_latent_attention(const Tensor& qa, const Tensor& cache, const Tensor& block_table, const Tensor& q_start,
+                           const Tensor& pos, const c10::optional<Tensor>& gate, double scale, int64_t rank,
+                           int64_t max_q) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(qa.device());
+    same_act(qa, cache, "latent_attention: queries and cache in one activation dtype");
+    need(qa.dim() == 3 && qa.is_contiguous() && cache.dim() == 3 && cache.is_contiguous(), "latent_attention: layouts");
+    const int64_t T = qa.size(0), H = qa.size(1), DK = qa.size(2);
+    need(cache.size(2) == DK && rank >= 1 && rank <= DK, "latent_attention: key width");
+    need(f32(qa) || DK % 2 == 0, "latent_attention: bf16 rows need an even width");
+    i32(block_table, "latent_attention: block_table"); i32(q_start, "latent_attention: q_start"); i32(pos, "latent_attention: pos");
+    const int64_t B = q_start.numel() - 1;
+    need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T, "latent_attention: metadata");
+    if (gate) { flt(*gate, "latent_attention: float32 gate"); need(gate->numel() == T * H, "latent_attention: gate [T, H]"); }
+    auto out = at::empty({T, H, rank}, qa.options());
+    if (T == 0 || B <= 0) return out;
+    const bool ok = chronos::launch_hy_latent_attention(
+        qa.data_ptr(), cache.data_ptr(), block_table.data_ptr<int32_t>(), (int)block_table.size(1),
+        q_start.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), gate ? gate->data_ptr<float>() : nullptr, out.data_ptr(),
+        (int)B, (int)H, (int)DK, (int)rank, (int)cache.size(1), (int)std::max<int64_t>(1, max_q), (float)scale, f32(qa),
+        stream());
+    TORCH_CHECK(ok, "chronos hybrid op: latent_attention has no launch geometry for heads=", H, " row width=", DK,
+                " rank=", rank, " (heads <= 64, rank <= 512, one key tile and the query rows must fit the LDS)");
+    return out;
+}
+
+std::tuple<Tensor, Tensor> hy_moe_route(const Tensor& h, const Tensor& w, const Tensor& corr, int64_t top) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w, "moe_route: h and router in one activation dtype");
+    need(h.dim() == 2 && w.dim() == 2 && h.is_contiguous() && w.is_contiguous() && h.size(1) == w.size(1), "moe_route: shapes");
+    flt(corr, "moe_route: float32 correction");
+    const int64_t N = w.size(0);
+    need(corr.numel() == N && N <= 256 && top >= 1 && top <= N, "moe_route: 1 <= top <= outputs <= 256");
+    auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
+    auto wt = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
+    chronos::launch_hy_moe_route(h.data_ptr(), w.data_ptr(), corr.data_ptr<float>(), idx.data_ptr<int32_t>(),
+                                 wt.data_ptr<float>(), (int)h.size(0), (int)h.size(1), (int)N, (int)top, f32(h), stream());
+    return {idx, wt};
+}
+
+Tensor hy_moe_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, const Tensor& w_up, const Tensor& w_down,
+                  int64_t act) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w_up, "moe_ffn: h and experts in one activation dtype");
+    same_act(h, w_down, "moe_ffn: h and experts in one activation dtype");
+    need(h.dim() == 2 && h.is_contiguous() && w_up.dim() == 3 && w_down.dim() == 3 && w_up.is_contiguous() && w_down.is_contiguous(), "moe_ffn: layouts");
+    const int64_t T = h.size(0), d = h.size(1), E = w_up.size(0), F = w_up.size(1);
+    need(w_up.size(2) == d && w_down.size(0) == E && w_down.size(1) == d && w_down.size(2) == F, "moe_ffn: expert shapes");
+    i32(idx, "moe_ffn: idx"); flt(wt, "moe_ffn: weights");
+    need(idx.dim() == 2 && idx.size(0) == T && wt.sizes() == idx.sizes(), "moe_ffn: idx / weights [T, top]");
+    need((2 * d + F) * 4 <= 160 * 1024, "moe_ffn: a token's rows must fit the LDS");
+    need(act == 0 || act == 1, "moe_ffn: activation kind");
+    auto out = at::empty_like(h);
+    chronos::launch_hy_moe_ffn_token(h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(), w_up.data_ptr(),
+                                     w_down.data_ptr(), out.data_ptr(), (int)T, (int)d, (int)F, (int)E, (int)idx.size(1),
+                                     (int)act, f32(h), stream());
+    return out;
+}
+
+}  // namespace
+
+TORCH_LIBRARY_FRAGMENT(chronos, m) {
+    m.def("hy_embed(Tensor ids, Tensor table) -> Tensor");
+    m.def("hy_cast_bf16(Tensor x) -> Tensor");
+    m.def("hy_layer_norm(Tensor x, Tensor w, float eps, bool out_f32) -> Tensor");
+    m.def("hy_add_layer_norm(Tensor y, Tensor(a!) x, Tensor w, float eps, bool out_f32) -> Tensor");
+    m.def("hy_rowdot(Tensor h, Tensor w, Tensor? bias) -> Tensor");
+    m.def("hy_act(Tensor(a!) x, int kind) -> ()");
+    m.def("hy_mlstm_scan(Tensor proj, Tensor gate_pre, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) S, "
+          "Tensor(b!) n, Tensor(c!) m, int H, int D, int Dv, float cap) -> Tensor");
+    m.def("hy_mlstm_out(Tensor o, Tensor proj, int g_off, Tensor w, float eps, bool out_f32) -> Tensor");
+    m.def("hy_latent_prep(Tensor(a!) q, Tensor dkv, Tensor pos, Tensor tok_seq, Tensor block_table, Tensor w_norm, "
+          "float eps, Tensor cos_sin, int dims, int rank, Tensor(b!) cache) -> ()");
+    m.def("hy_latent_attention(Tensor qa, Tensor cache, Tensor block_table, Tensor q_start, Tensor pos, Tensor? gate, "
+          "float scale, int rank, int max_q) -> Tensor");
+    m.def("hy_moe_route(Tensor h, Tensor w, Tensor corr, int top) -> (Tensor, Tensor)");
+    m.def("hy_moe_ffn(Tensor h, Tensor idx, Tensor wt, Tensor w_up, Tensor w_down, int act) -> Tensor");
+}
+
+TORCH_LIBRARY_IMPL(chronos, CUDA, m) {
+    m.impl("hy_embed", &hy_embed);
+    m.impl("hy_cast_bf16", &hy_cast_bf16);
+    m.impl("hy_layer_norm", &hy_layer_norm);
+    m.impl("hy_add_layer_norm", &hy_add_layer_norm);
+    m.impl("hy_rowdot", &hy_rowdot);
+    m.impl("hy_act", &hy_act);
+    m.impl("hy_mlstm_scan", &hy_mlstm_scan);
+    m.impl("hy_mlstm_out", &hy_mlstm_out);
+    m.impl("hy_latent_prep", &hy_latent_prep);
+    m.impl("hy_latent_attention", &hy_latent_attention);
+    m.impl("hy_moe_route", &hy_moe_route);
+    m.impl("hy_moe_ffn", &hy_moe_ffn);
+}

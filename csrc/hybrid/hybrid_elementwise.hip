@@ -1,0 +1,120 @@
+// hybrid_elementwise.hip — the float32 residual stream of the hybrid decoders: embedding rows, layer norm (weight, no
+// bias) with the residual add fused, the few-row float32-output projections, activations.
+//
+// The sublayers' outputs are normalised and ADDED to the stream (x <- x + norm(y)), so the norm kernel reads the
+// sublayer output in the activation type, does all its arithmetic in float, updates the float stream in place and
+// emits the stream's copy in the activation type for the next sublayer's GEMMs (one pass, nothing re-read from HBM).
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+template <typename T>
+__global__ void __launch_bounds__(256) embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+                                                    float* __restrict__ x, int d) {
+    const int64_t t = blockIdx.x;
+    const T* src = table + (int64_t)ids[t] * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) x[t * d + i] = ld<T>(src + i);
+}
+
+__global__ void __launch_bounds__(256) cast_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i + 3 < n) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(x + i);
+        *reinterpret_cast<u16x4*>(y + i) = u16x4{f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+    } else {
+        for (int64_t j = i; j < n; ++j) y[j] = f2bf(x[j]);
+    }
+}
+
+// y [rows, d] (activation type, or float for the plain norm of the stream itself) -> float statistics in two passes
+// (mean, then the mean of squared deviations), then
+//   ADD:   x[row] += (y - mean) * rstd * w;   h[row] = T(x[row])   (h == nullptr: not written)
+//   plain: h[row] = T((y - mean) * rstd * w)
+template <typename TY, typename TH, bool ADD>
+__global__ void __launch_bounds__(256) layer_norm_kernel(const TY* __restrict__ y, float* __restrict__ x,
+                                                         const float* __restrict__ w, TH* __restrict__ h, int d,
+                                                         float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    const TY* yr = y + row * d;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < d; i += 256) s += ld<TY>(yr + i);
+    const float mean = block_sum(s, red) / (float)d;
+    float q = 0.f;
+    for (int i = threadIdx.x; i < d; i += 256) {
+        const float c = ld<TY>(yr + i) - mean;
+        q += c * c;
+    }
+    const float rstd = 1.f / sqrtf(block_sum(q, red) / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += 256) {
+        float v = (ld<TY>(yr + i) - mean) * rstd * w[i];
+        if constexpr (ADD) {
+            v += x[row * d + i];
+            x[row * d + i] = v;
+        }
+        if (h != nullptr) st<TH>(h + row * d + i, v);
+    }
+}
+
+// out[t, n] = sum_k h[t, k] * w[n, k] (+ bias[n]) in float: one workgroup per token, one wave per output row in turn.
+template <typename T>
+__global__ void __launch_bounds__(256) rowdot_kernel(const T* __restrict__ h, const T* __restrict__ w,
+                                                     const float* __restrict__ bias, float* __restrict__ out, int d,
+                                                     int n) {
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const T* hr = h + t * d;
+    for (int r = wv; r < n; r += 4) {
+        const T* wr = w + (int64_t)r * d;
+        float acc = 0.f;
+        for (int k = lane; k < d; k += 64) acc += ld<T>(hr + k) * ld<T>(wr + k);
+        acc = wave_sum(acc);
+        if (lane == 0) out[t * n + r] = acc + (bias != nullptr ? bias[r] : 0.f);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) act_kernel(T* __restrict__ x, int64_t n, int kind) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) st<T>(x + i, act_apply(ld<T>(x + i), kind));
+}
+
+}  // namespace hy
+
+void launch_hy_embed(const int32_t* ids, const void* table, float* x, int T, int d, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    if (f32) hy::embed_kernel<float><<<T, 256, 0, s>>>(ids, (const float*)table, x, d);
+    else hy::embed_kernel<uint16_t><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, x, d);
+}
+void launch_hy_cast_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t s) {
+    if (n == 0) return;
+    const int64_t blocks = (n + 1023) / 1024;
+    hy::cast_bf16_kernel<<<(unsigned)blocks, 256, 0, s>>>(x, y, n);
+}
+// y_f32: the input is float (the plain norm of the stream); out_f32: h is float.  x == nullptr: plain norm.
+void launch_hy_layer_norm(const void* y, bool y_f32, float* x, const float* w, void* h, bool out_f32, int rows, int d,
+                          float eps, hipStream_t s) {
+    if (rows == 0) return;
+    if (x != nullptr) {
+        if (y_f32) hy::layer_norm_kernel<float, float, true><<<rows, 256, 0, s>>>((const float*)y, x, w, (float*)h, d, eps);
+        else hy::layer_norm_kernel<uint16_t, uint16_t, true><<<rows, 256, 0, s>>>((const uint16_t*)y, x, w, (uint16_t*)h, d, eps);
+    } else {
+        if (out_f32) hy::layer_norm_kernel<float, float, false><<<rows, 256, 0, s>>>((const float*)y, nullptr, w, (float*)h, d, eps);
+        else hy::layer_norm_kernel<float, uint16_t, false><<<rows, 256, 0, s>>>((const float*)y, nullptr, w, (uint16_t*)h, d, eps);
+    }
+}
+void launch_hy_rowdot(const void* h, const void* w, const float* bias, float* out, int T, int d, int n, bool f32,
+                      hipStream_t s) {
+    if (T == 0 || n == 0) return;
+    if (f32) hy::rowdot_kernel<float><<<T, 256, 0, s>>>((const float*)h, (const float*)w, bias, out, d, n);
+    else hy::rowdot_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)h, (const uint16_t*)w, bias, out, d, n);
+}
+void launch_hy_act(void* x, int64_t n, int kind, bool f32, hipStream_t s) {
+    if (n == 0) return;
+    const int64_t blocks = (n + 255) / 256;
+    if (f32) hy::act_kernel<float><<<(unsigned)blocks, 256, 0, s>>>((float*)x, n, kind);
+    else hy::act_kernel<uint16_t><<<(unsigned)blocks, 256, 0, s>>>((uint16_t*)x, n, kind);
+}
+
+}  // namespace chronos

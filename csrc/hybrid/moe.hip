@@ -1,0 +1,157 @@
+// moe.hip — mixture-of-experts feed-forward of the hybrid decoders.
+//
+//   route   per token: float router logits (N = experts + identity outputs), softmax over all N, the `top` largest
+//           of score + correction chosen (the correction steers the choice only), weights = the chosen outputs' plain
+//           scores, not renormalised.  Ties go to the lower index.
+//   ffn     per token: sum over its chosen experts of weight * W_down act(W_up h); an index >= E is an identity
+//           expert (weight * h).  Token-parallel form: one workgroup per token streams the chosen experts' weights
+//           (the decode regime: few tokens, every expert matrix read about once; float accumulation throughout).
+//
+// No step of either kernel depends on the host knowing the routing: both capture into a graph.
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+constexpr int kMaxRouterOut = 256;  // N <= 256 (4 per lane)
+
+template <typename T>
+__global__ void __launch_bounds__(256) moe_route_kernel(const T* __restrict__ h, const T* __restrict__ w,
+                                                        const float* __restrict__ corr, int32_t* __restrict__ idx,
+                                                        float* __restrict__ wt, int d, int N, int top) {
+    __shared__ float z[kMaxRouterOut];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const T* hr = h + t * d;
+    for (int r = wv; r < N; r += 4) {
+        const T* wr = w + (int64_t)r * d;
+        float acc = 0.f;
+        for (int k = lane; k < d; k += 64) acc += ld<T>(hr + k) * ld<T>(wr + k);
+        acc = wave_sum(acc);
+        if (lane == 0) z[r] = acc;
+    }
+    __syncthreads();
+    if (wv != 0) return;
+    float s[4], c[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        s[j] = e < N ? z[e] : -INFINITY;
+        mx = fmaxf(mx, s[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s[j] = (lane + 64 * j < N) ? expf(s[j] - mx) : 0.f;
+        sum += s[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        s[j] = s[j] / sum;
+        c[j] = e < N ? s[j] + corr[e] : -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) {
+        // the wave's best (value, lowest index): a lane's own candidates first, then across lanes
+        float bv = -INFINITY, bs = 0.f;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = lane + 64 * j;
+            if (c[j] > bv || (c[j] == bv && e < be && c[j] != -INFINITY)) {
+                bv = c[j]; be = e; bs = s[j];
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64), os = __shfl_xor(bs, o, 64);
+            const int oe = __shfl_xor(be, o, 64);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov; be = oe; bs = os;
+            }
+        }
+        if (lane == 0) {
+            idx[t * top + k] = be;
+            wt[t * top + k] = bs;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (lane + 64 * j == be) c[j] = -INFINITY;
+    }
+}
+
+// LDS: h row (d floats) | z (F floats) | out (d floats).
+template <typename T>
+__global__ void __launch_bounds__(256) moe_ffn_token_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
+                                                            const float* __restrict__ wt, const T* __restrict__ w_up,
+                                                            const T* __restrict__ w_down, T* __restrict__ out, int d,
+                                                            int F, int E, int top, int act) {
+    extern __shared__ float sm[];
+    float* hs = sm;
+    float* zs = hs + d;
+    float* os = zs + F;
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < d; i += 256) {
+        hs[i] = ld<T>(h + t * d + i);
+        os[i] = 0.f;
+    }
+    __syncthreads();
+    for (int k = 0; k < top; ++k) {
+        const int e = idx[t * top + k];
+        const float g = wt[t * top + k];
+        if (e >= E) {  // identity expert (uniform over the workgroup)
+            for (int i = threadIdx.x; i < d; i += 256) os[i] += g * hs[i];
+            __syncthreads();
+            continue;
+        }
+        const T* wu = w_up + (int64_t)e * F * d;
+        for (int f = wv; f < F; f += 4) {
+            const T* wr = wu + (int64_t)f * d;
+            float acc = 0.f;
+            for (int i = lane; i < d; i += 64) acc += ld<T>(wr + i) * hs[i];
+            acc = wave_sum(acc);
+            if (lane == 0) zs[f] = act_apply(rnd<T>(acc), act);
+        }
+        __syncthreads();
+        const T* wd = w_down + (int64_t)e * d * F;
+        for (int r = wv; r < d; r += 4) {
+            const T* wr = wd + (int64_t)r * F;
+            float acc = 0.f;
+            for (int i = lane; i < F; i += 64) acc += ld<T>(wr + i) * zs[i];
+            acc = wave_sum(acc);
+            if (lane == 0) os[r] += g * acc;
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < d; i += 256) st<T>(out + t * d + i, os[i]);
+}
+
+}  // namespace hy
+
+void launch_hy_moe_route(const void* h, const void* w, const float* corr, int32_t* idx, float* wt, int T, int d, int N,
+                         int top, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    if (f32) hy::moe_route_kernel<float><<<T, 256, 0, s>>>((const float*)h, (const float*)w, corr, idx, wt, d, N, top);
+    else hy::moe_route_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)h, (const uint16_t*)w, corr, idx, wt, d, N, top);
+}
+
+void launch_hy_moe_ffn_token(const void* h, const int32_t* idx, const float* wt, const void* w_up, const void* w_down,
+                             void* out, int T, int d, int F, int E, int top, int act, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    const int bytes = (2 * d + F) * 4;
+    if (f32) {
+        auto kern = hy::moe_ffn_token_kernel<float>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<T, 256, bytes, s>>>((const float*)h, idx, wt, (const float*)w_up, (const float*)w_down, (float*)out, d, F, E, top, act);
+    } else {
+        auto kern = hy::moe_ffn_token_kernel<uint16_t>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<T, 256, bytes, s>>>((const uint16_t*)h, idx, wt, (const uint16_t*)w_up, (const uint16_t*)w_down, (uint16_t*)out, d, F, E, top, act);
+    }
+}
+
+}  // namespace chronos

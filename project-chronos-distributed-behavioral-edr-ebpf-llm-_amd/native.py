@@ -6,6 +6,8 @@ to the GPU box and show up as in-tree loads):
   _sensor_native   g++      csrc/sensor_host/*.cpp      shared eBPF filter policy, data_t codec, chain tracker
   _constrain_native g++     csrc/constrain/*.cpp        JSON / verdict-schema token automaton compiler, tokenizer trie
   _C               hipcc    csrc/kernels/*.hip          gfx950 HIP kernels (MFMA/LDS) as torch ops
+  _H               hipcc    csrc/hybrid/*.hip           the hybrid-decoder kernels (recurrent state, latent attention,
+                                                        mixture of experts) as torch ops, loadable without _C
 
 The HIP library is compiled with hipcc directly (``--offload-arch=gfx950``), not through torch's cpp_extension, so no
 hipify pass ever touches the sources.  Rebuilds are keyed on a hash of sources + flags.
@@ -180,6 +182,8 @@ def hip_flags() -> tuple[list[str], list[str]]:
         "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
         "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1", "-Wno-unused-result", "-Wno-deprecated-declarations",
         "-Wno-unused-command-line-argument",
+        # no packed-fp32 VALU forms (v_pk_*_f32) from ordinary float code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         f"-I{os.path.join(CSRC, 'include')}",
     ] + [f"-I{i}" for i in incs] + [f"-I{sysconfig.get_paths()['include']}"]
     if os.environ.get("CHRONOS_GEMM_ABLATIONS") == "1":  # diagnostics build: gemm_lg's timing-only ablation ids
@@ -197,9 +201,19 @@ def build_kernels(force: bool = False, jobs: int = 8) -> str:
     return _build("_C", srcs, [hipcc], cflags, ldflags, deps, force, jobs)
 
 
+def build_hybrid(force: bool = False, jobs: int = 8) -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    srcs = sorted(glob.glob(os.path.join(CSRC, "hybrid", "*.hip")) + glob.glob(os.path.join(CSRC, "hybrid", "*.cpp")))
+    cflags, ldflags = hip_flags()
+    cflags = [f.replace("-DTORCH_EXTENSION_NAME=_C", "-DTORCH_EXTENSION_NAME=_H") for f in cflags]
+    deps = _deps([os.path.join(CSRC, "hybrid"), os.path.join(CSRC, "include")])
+    return _build("_H", srcs, [hipcc], cflags, ldflags, deps, force, jobs)
+
+
 def build_all(force: bool = False) -> None:
     build_sensor(force)
     build_constrain(force)
+    build_hybrid(force)
     build_kernels(force)
 
 
@@ -222,6 +236,20 @@ def sensor_lib():
 
 def constrain_lib():
     return _import_built("_constrain_native", build_constrain)
+
+
+def hybrid_lib():
+    """Load the hybrid-decoder kernel library (registers torch.ops.chronos.hy_*).  Builds it in-tree if stale."""
+    with _lock:
+        if "_H" in _loaded:
+            return _loaded["_H"]
+    import torch  # noqa: F401
+
+    path = build_hybrid()
+    with _lock:
+        torch.ops.load_library(path)
+        _loaded["_H"] = path
+    return path
 
 
 def kernels_lib():

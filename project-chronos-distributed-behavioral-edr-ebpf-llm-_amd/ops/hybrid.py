@@ -1,5 +1,5 @@
 """Ops of the hybrid decoders (recurrent matrix-memory layers, latent attention, mixtures of experts, layer norms on
-a float32 residual stream): gfx950 HIP kernels on the GPU (csrc/kernels/hybrid_*.hip), the PyTorch references of
+a float32 residual stream): gfx950 HIP kernels on the GPU (csrc/hybrid/*.hip), the PyTorch references of
 :mod:`.hybrid_ref` on the CPU.
 
 As everywhere in :mod:`chronos.ops` a GPU tensor never falls back silently: it goes to ``torch.ops.chronos.hy_*`` or
@@ -25,10 +25,22 @@ def _gpu(t: torch.Tensor) -> bool:
     return t.is_cuda and not _REF_ON_GPU
 
 
-def _k():
-    from . import _k as k
+_lib_loaded = False
 
-    return k()
+
+def load() -> None:
+    """Load (building in-tree if stale) the hybrid kernel library; raises on failure."""
+    global _lib_loaded
+    if not _lib_loaded:
+        from ..native import hybrid_lib
+
+        hybrid_lib()
+        _lib_loaded = True
+
+
+def _k():
+    load()
+    return torch.ops.chronos
 
 
 def _f32(act_dtype) -> bool:

@@ -1,0 +1,324 @@
+"""Zokunex through the framework (registry -> engine -> block manager / state slots -> step batches -> ops) against
+the plain token-by-token oracle of tests/oracles/zokunex_plain.py.
+
+CPU runs take the ops' PyTorch path, the ``cuda`` parametrisations (marked gpu) the HIP kernels; both go through the
+same engine code.  Sizes are deliberately unlike each other (head counts 1-3, widths that are no tile multiples, rotated
+columns fewer than the rotated part, routers with and without identity experts, top 1).
+"""
+import copy
+import json
+
+import pytest
+import torch
+
+from tests.oracles import zokunex_plain as plain
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+
+
+def _mlstm(heads=3, dim=8, vdim=12, cap=10.0):
+    return dict(type="mlstm", mixer=dict(heads=heads, dim=dim, vdim=vdim, gate_cap=cap))
+
+
+def _latent(heads=2, dim=8, rot_dim=12, dims=8, vdim=20, rank=16, scale=0.2, base=5000.0):
+    return dict(type="latent_attention", mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=rank,
+                                                    scale=scale, rot=dict(base=base, dims=dims)))
+
+
+def _dense(ff=40):
+    return dict(kind="dense", ff=ff)
+
+
+def _moe(experts=3, identity=2, top=2, ff=24):
+    return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, identity=identity, top=top))
+
+
+def _config(layers, width=64, vocab=97, logit_scale=0.5, eps=1e-5):
+    return dict(architecture="Zokunex", vocab=vocab, width=width, logit_scale=logit_scale, norm=dict(eps=eps),
+                layers=[dict(l[0], mlp=l[1]) for l in layers])
+
+
+MIXED = _config([(_mlstm(), _moe()), (_latent(), _dense()), (_latent(heads=1, dim=4, rot_dim=4, dims=4, vdim=8, rank=24), None),
+                 (_mlstm(heads=1, dim=20, vdim=70, cap=4.0), _dense(24)), (_mlstm(heads=2, dim=6, vdim=6), _moe(1, 0, 1, 16)),
+                 (_latent(heads=3, dim=12, rot_dim=6, dims=6, vdim=4, rank=10, scale=0.6, base=300.0), _moe(4, 3, 4, 8))])
+
+
+def _model(cfg_dict, device, dtype="fp32", seed=0, tensors=None):
+    from chronos.models import zokunex
+
+    cfg = zokunex.config_from_dict(cfg_dict, max_position=1024)
+    if tensors is None:
+        tensors = zokunex.random_tensors(cfg, seed)
+        if dtype == "bf16":  # routers far from close calls: a choice flipped by rounding would feed the recurrent
+            for k in tensors:  # state and move every later position of the request
+                if k.endswith("mlp.router"):
+                    tensors[k] = tensors[k] * 8
+    at = torch.float32 if dtype == "fp32" else torch.bfloat16
+    from chronos.models.hybrid import HybridDecoder
+
+    return HybridDecoder(cfg, zokunex.pack_weights(cfg, tensors, device, at), device, 1024, at), tensors
+
+
+def _engine(cfg_dict, device, dtype="fp32", slots=4, max_len=512, blocks=0, seed=0, tensors=None, **kw):
+    from chronos.brain.engine.engine import Engine, EngineConfig
+
+    model, tensors = _model(cfg_dict, device, dtype, seed, tensors)
+    bs = kw.pop("block_size", 16)
+    ec = EngineConfig(model="zokunex-test", device=device, dtype=dtype, max_slots=slots, block_size=bs,
+                      max_model_len=max_len, kv_blocks=blocks or slots * (max_len // bs) + 1, warm_formats=(), **kw)
+    return Engine(ec, model=model), tensors
+
+
+def _errs(got, want):
+    """Per position: the spread of the difference over the vocabulary relative to the spread of the logits."""
+    d = got.double() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def _err(got, want):
+    return float(_errs(got, want).max())
+
+
+def _bad(got, want, dtype):
+    """float32: the worst position against the tolerance.  bfloat16: rounding can flip a close router choice at a
+    single position of these tiny random models, so the 85th percentile of the positions is held to the tolerance
+    (a fault of a mechanism, a cache or a schedule moves far more positions than that)."""
+    e = _errs(got, want)
+    if dtype == "fp32" or e.numel() < 8:
+        return float(e.max()) >= TOL[dtype] * (1 if dtype == "fp32" else 4)
+    return float(e.sort().values[int(0.85 * (e.numel() - 1))]) >= TOL[dtype]
+
+
+def _tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def _replay(eng, schedule, reqs):
+    """schedule: list of steps, each [(request name, count)].  Returns {name: logits of every token}."""
+    from chronos.brain.engine.replay import TraceSession
+
+    ses = TraceSession(eng)
+    at = {k: 0 for k in reqs}
+    out = {k: [] for k in reqs}
+    for step in schedule:
+        entries, end = [], []
+        for name, count in step:
+            lo = at[name]
+            entries.append(dict(id=name, tokens=reqs[name][lo:lo + count], want=list(range(count))))
+            at[name] = lo + count
+            if at[name] == len(reqs[name]):
+                end.append(name)
+        logits = ses.step(entries, end)
+        k = 0
+        for name, count in step:
+            out[name].append(logits[k:k + count])
+            k += count
+    assert not ses.live
+    return {k: torch.cat(v) for k, v in out.items()}
+
+
+TOL = {"fp32": 2e-4, "bf16": 0.1}
+
+
+# ---- each mechanism alone, layer by layer -------------------------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("layer", [(_mlstm(), None), (_mlstm(heads=1, dim=5, vdim=3, cap=2.0), None), (_latent(), None),
+                                   (_latent(heads=1, dim=2, rot_dim=2, dims=2, vdim=2, rank=2, scale=1.5), None),
+                                   (_mlstm(), _dense()), (_mlstm(), _moe()), (_mlstm(), _moe(2, 0, 2, 8)),
+                                   (_latent(), _moe(1, 3, 2, 8))])
+def test_single_layer_and_residual_stream(device, layer):
+    cfg = _config([layer, layer])
+    model, tensors = _model(cfg, device)
+    toks = _tokens(37, cfg["vocab"], 3)
+    taps = []
+    model.layer_tap = lambda li, x: taps.append(x.detach().clone().cpu())
+    cache = model.make_cache(8, 16, 2)
+    sb = model.prefill_batch([toks], [0], [[1, 2, 3]], [1], want=list(range(len(toks))))
+    got = model.forward(sb, cache).cpu()
+    per_layer = []
+    want = plain.forward(cfg, tensors, toks, layers_out=per_layer)
+    for li, x in enumerate(taps):
+        assert float((x.double() - per_layer[li]).abs().max()) < 2e-4 * float(per_layer[li].abs().max()), f"layer {li}"
+    assert _err(got, want) < TOL["fp32"]
+
+
+# ---- schedules: whole prompts, decoding, portions, mixed batches ---------------------------------------------------
+def _requests(cfg, lens, seed=0):
+    return {f"r{i}": _tokens(n, cfg["vocab"], seed + i) for i, n in enumerate(lens)}
+
+
+def _check(eng, tensors, cfg, schedule, reqs, dtype):
+    got = _replay(eng, schedule, reqs)
+    for name, toks in reqs.items():
+        want = plain.forward(cfg, tensors, toks)
+        assert not _bad(got[name].cpu(), want, dtype), (name, _errs(got[name].cpu(), want))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_prefill_equals_token_by_token(device, dtype):
+    eng, tensors = _engine(MIXED, device, dtype)
+    reqs = _requests(MIXED, [45, 1, 18])
+    sched = [[("r0", 45)], [("r1", 1)]] + [[("r2", 1)] for _ in range(18)]
+    _check(eng, tensors, MIXED, sched, reqs, dtype)
+    # the same prompt once more, most of it at once and the rest decoded: the slot and pages are reused
+    sched = [[("r0", 13)]] + [[("r0", 1)] for _ in range(32)]
+    _check(eng, tensors, MIXED, sched, {"r0": reqs["r0"]}, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_portions_of_every_size(device):
+    eng, tensors = _engine(MIXED, device)
+    reqs = _requests(MIXED, [100], seed=5)
+    cuts = [3, 2, 16, 2, 15, 17, 2, 31, 1, 1, 2, 7, 1]
+    assert sum(cuts) == 100
+    _check(eng, tensors, MIXED, [[("r0", c)] for c in cuts], reqs, "fp32")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_mixed_batches_with_reused_pages_and_slots(device, dtype):
+    """Four slots and a pool of 14 pages (block 0 is scratch) for six requests of 212 tokens in all: requests end,
+    their pages and slots go to new ones; portions run beside single decoded tokens."""
+    eng, tensors = _engine(MIXED, device, dtype, slots=4, max_len=128, blocks=15)
+    reqs = _requests(MIXED, [70, 9, 33, 1, 40, 59], seed=11)
+    sched = [[("r0", 3), ("r1", 1)],
+             [("r0", 30), ("r1", 1), ("r2", 2)],
+             [("r0", 1), ("r1", 2), ("r2", 29), ("r3", 1)],
+             [("r0", 1), ("r1", 1), ("r2", 1), ("r4", 17)],
+             [("r0", 16), ("r1", 4), ("r2", 1), ("r4", 1)],      # r1, r2 end
+             [("r0", 1), ("r4", 1), ("r5", 2)],
+             [("r0", 18), ("r4", 21), ("r5", 31)],               # r0, r4 end
+             [("r5", 1)]] + [[("r5", 1)] for _ in range(25)]
+    _check(eng, tensors, MIXED, sched, reqs, dtype)
+    assert eng.blocks.free == 14 and len(eng.free_slots) == 4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batch_members_do_not_see_each_other(device):
+    eng, tensors = _engine(MIXED, device)
+    reqs = _requests(MIXED, [21, 64, 5], seed=21)
+    alone = {k: _replay(eng, [[(k, len(v))]], {k: v})[k] for k, v in reqs.items()}
+    together = _replay(eng, [[("r0", 21), ("r1", 64), ("r2", 5)]], reqs)
+    for k in reqs:
+        assert _err(together[k], alone[k]) < 1e-5
+
+
+# ---- keys far away and at the causal edge; page borders -----------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decode", [False, True])
+def test_far_key_dominates(device, decode):
+    """Latent attention with a sharp softmax (large scale): the answer at the end hangs on single keys hundreds of
+    tokens back, across many pages; a lost page or an off-by-one in the visible range changes the logits."""
+    cfg = _config([(_latent(heads=2, dim=8, rot_dim=4, dims=4, vdim=8, rank=16, scale=6.0), None)], width=32)
+    eng, tensors = _engine(cfg, device, max_len=640)
+    toks = _tokens(600, cfg["vocab"], 2)
+    sched = [[("r0", 590)]] + [[("r0", 1)] for _ in range(10)] if decode else [[("r0", 33)], [("r0", 567)]]
+    got = _replay(eng, sched, {"r0": toks})["r0"]
+    want = plain.forward(cfg, tensors, toks, want=range(560, 600))
+    assert _err(got[560:].cpu(), want) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_causal_edge_at_page_borders(device):
+    """Every position from just before a page border to just after it, decoded and in portions that start and end at
+    the border, with a sharp softmax."""
+    cfg = _config([(_latent(scale=4.0), _dense()), (_mlstm(), None)], width=48)
+    eng, tensors = _engine(cfg, device, block_size=16)
+    toks = _tokens(52, cfg["vocab"], 8)
+    want = plain.forward(cfg, tensors, toks)
+    for sched in ([[("r0", 14)]] + [[("r0", 1)] for _ in range(38)],
+                  [[("r0", 16)], [("r0", 16)], [("r0", 15)], [("r0", 2)], [("r0", 3)]],
+                  [[("r0", 15)], [("r0", 2)], [("r0", 30)], [("r0", 5)]]):
+        assert _err(_replay(eng, sched, {"r0": toks})["r0"].cpu(), want) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_recurrent_state_saturating_gates(device):
+    """Gate pre-activations far beyond the cap on both sides (forget gate shut / wide open, input gate huge): the
+    running maximum has to carry the scale; the state is carried over 3 portions and 40 decoded tokens."""
+    from chronos.models import zokunex
+
+    cfg = _config([(_mlstm(heads=2, dim=8, vdim=8, cap=15.0), None), (_mlstm(heads=1, dim=4, vdim=16, cap=3.0), _dense())], width=32)
+    t = zokunex.random_tensors(zokunex.config_from_dict(cfg), 4)
+    t["l0.mix.i"] = t["l0.mix.i"] * 60
+    t["l0.mix.f"] = t["l0.mix.f"] * 60
+    t["l0.mix.f.b"] = torch.tensor([-20.0, 20.0]).to(torch.bfloat16)
+    t["l1.mix.i.b"] = torch.tensor([9.0]).to(torch.bfloat16)
+    eng, tensors = _engine(cfg, device, tensors=t)
+    toks = _tokens(90, cfg["vocab"], 6)
+    sched = [[("r0", 7)], [("r0", 2)], [("r0", 41)]] + [[("r0", 1)] for _ in range(40)]
+    assert _err(_replay(eng, sched, {"r0": toks})["r0"].cpu(), plain.forward(cfg, tensors, toks)) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_router_correction_steers_choice_only(device):
+    """A correction that lifts the weakest outputs above the strongest: the chosen set follows score + correction,
+    the weights stay the plain scores (an identity expert among them)."""
+    from chronos.models import zokunex
+
+    cfg = _config([(_mlstm(), _moe(3, 2, 2, 16))], width=32)
+    t = zokunex.random_tensors(zokunex.config_from_dict(cfg), 9)
+    t["l0.mlp.correction"] = torch.tensor([0.0, 5.0, 0.0, 0.0, 4.0]).to(torch.bfloat16)
+    eng, tensors = _engine(cfg, device, tensors=t)
+    toks = _tokens(20, cfg["vocab"], 1)
+    assert _err(_replay(eng, [[("r0", 20)]], {"r0": toks})["r0"].cpu(), plain.forward(cfg, tensors, toks)) < TOL["fp32"]
+    t2 = dict(t)
+    t2["l0.mlp.correction"] = torch.zeros(5).to(torch.bfloat16)
+    assert _err(plain.forward(cfg, t2, toks), plain.forward(cfg, tensors, toks)) > 1e-2, "the test must be sensitive"
+
+
+# ---- generation through the engine's own entry point and scheduler ------------------------------------------------
+def _greedy(cfg, tensors, prompt, n):
+    ids = list(prompt)
+    for _ in range(n):
+        ids.append(int(plain.forward(cfg, tensors, ids, want=[len(ids) - 1])[0].argmax()))
+    return ids[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(device, graphs):
+    """submit() -> admission -> prefill / mixed steps -> decode bursts -> harvest, five requests over two slots and a
+    small page pool (slots and pages are reused, arrivals join running decodes), greedy tokens equal to the oracle's."""
+    if graphs and device == "cpu":
+        pytest.skip("graphs are a GPU feature")
+    cfg = _config([(_mlstm(heads=2, dim=8, vdim=8), _moe(3, 1, 2, 16)), (_latent(), _dense(32))], width=32, vocab=61, logit_scale=4.0)
+    eng, tensors = _engine(cfg, device, slots=2, max_len=96, blocks=9, use_graphs=graphs, decode_burst=4,
+                           max_prefill_tokens=24, mixed_prefill_tokens=8, prefill_ramp=0)
+    prompts = [_tokens(n, 59, 30 + n) for n in (5, 31, 12, 2, 40)]   # (ids 59 and 60 are the byte tokenizer's specials)
+    reqs = [eng.submit(p, num_predict=9) for p in prompts[:3]]
+    eng.step()
+    eng.step()
+    reqs += [eng.submit(p, num_predict=9) for p in prompts[3:]]
+    eng.run_until_idle(max_steps=2000)
+    for r, p in zip(reqs, prompts):
+        assert r.done_reason in ("length", "stop"), (r.done_reason, r.error)
+        want = _greedy(cfg, tensors, p, 9)
+        n = len(r.out_ids)
+        # (the engine's free-text automaton spends the last token of the budget on the end-of-text token)
+        assert n >= 8 and r.out_ids == want[:n], (r.out_ids, want)
+    assert eng.blocks.free == 8 and len(eng.free_slots) == 2
+
+
+def test_registry_reads_the_checkpoint_layout(tmp_path):
+    from chronos.models import registry, zokunex
+
+    cfg = zokunex.config_from_dict(MIXED)
+    tensors = zokunex.random_tensors(cfg, 1)
+    zokunex.save(cfg, tensors, str(tmp_path))
+    assert json.load(open(tmp_path / "config.json"))["layers"] == zokunex.config_to_dict(cfg)["layers"]
+    assert registry.family_of(str(tmp_path)).name == "zokunex"
+    model = registry.build_model(str(tmp_path), "cpu", dtype="fp32", max_position=64)
+    toks = _tokens(9, cfg.vocab_size, 0)
+    sb = model.prefill_batch([toks], [0], [[1]], [0], want=list(range(9)))
+    assert _err(model.forward(sb, model.make_cache(2, 16, 1)), plain.forward(MIXED, tensors, toks)) < TOL["fp32"]
+    bad = copy.deepcopy(MIXED)
+    bad["layers"][0]["type"] = "conv"
+    with pytest.raises(ValueError):
+        zokunex.config_from_dict(bad)
+    with pytest.raises(NotImplementedError):
+        registry.build_model("tiny", "cpu", dtype="fp32")
