@@ -84,6 +84,10 @@ def parse():
     ap.add_argument("--max-model-len", type=int, default=512)
     ap.add_argument("--sequence-parallel", action="store_true",
                     help="with --tp: Megatron sequence parallelism in prefill (reduce-scatter / all-gather)")
+    ap.add_argument("--design-compare", action="store_true",
+                    help="instead of the headline: prefill / decode throughput of the Zokunex hybrid design beside "
+                         "Llama at equal width and depth, and its kernels beside their Llama counterparts")
+    ap.add_argument("--design-sizes", default="1k,2k,4k", help="with --design-compare: widths to measure")
     return ap.parse_args()
 
 
@@ -172,6 +176,10 @@ def ensure_world(a) -> int | None:
 
 def main():
     a = parse()
+    if a.design_compare:
+        from chronos.utils import design_bench
+
+        return design_bench.main(a)
     rc = ensure_world(a)
     if rc is not None:
         return rc
