@@ -30,6 +30,9 @@ void launch_hy_moe_route(const void*, const void*, const float*, int32_t*, float
                          hipStream_t);
 void launch_hy_moe_ffn_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
                              int, int, int, bool, hipStream_t);
+int hy_moe_max_tiles(int, int);
+void launch_hy_moe_grouped(const uint16_t*, const int32_t*, const float*, const uint16_t*, const uint16_t*, uint16_t*,
+                           int32_t*, uint16_t*, uint16_t*, int, int, int, int, int, int, hipStream_t);
 }  // namespace chronos
 
 namespace {
@@ -219,6 +222,20 @@ Tensor hy_moe_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, const Te
     need((2 * d + F) * 4 <= 160 * 1024, "moe_ffn: a token's rows must fit the LDS");
     need(act == 0 || act == 1, "moe_ffn: activation kind");
     auto out = at::empty_like(h);
+    // bfloat16 with tile-sized widths: the grouped MFMA GEMMs (each expert's weights once per 128 of its tokens);
+    // float32, or widths off the 128 grid: the token-parallel kernel
+    if (!f32(h) && d % 128 == 0 && F % 128 == 0 && E <= 256 && T > 0) {
+        const int top = (int)idx.size(1), items = (int)T * top;
+        const int maxTiles = chronos::hy_moe_max_tiles(items, (int)E);
+        auto meta = at::empty({1 + (int64_t)maxTiles + (int64_t)maxTiles * 128 + items}, h.options().dtype(at::kInt));
+        auto z = at::empty({(int64_t)maxTiles * 128, F}, h.options());
+        auto yrows = at::empty({(int64_t)maxTiles * 128, d}, h.options());
+        chronos::launch_hy_moe_grouped((const uint16_t*)h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(),
+                                       (const uint16_t*)w_up.data_ptr(), (const uint16_t*)w_down.data_ptr(),
+                                       (uint16_t*)out.data_ptr(), meta.data_ptr<int32_t>(), (uint16_t*)z.data_ptr(),
+                                       (uint16_t*)yrows.data_ptr(), (int)T, (int)d, (int)F, (int)E, top, (int)act, stream());
+        return out;
+    }
     chronos::launch_hy_moe_ffn_token(h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(), w_up.data_ptr(),
                                      w_down.data_ptr(), out.data_ptr(), (int)T, (int)d, (int)F, (int)E, (int)idx.size(1),
                                      (int)act, f32(h), stream());

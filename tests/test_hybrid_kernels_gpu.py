@@ -190,12 +190,14 @@ def test_latent_attention_sees_exactly_its_prefix(dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("d,F,E,I,top", [(256, 64, 8, 4, 3), (96, 40, 3, 0, 1), (128, 200, 5, 2, 7)])
-def test_moe(dt, d, F, E, I, top):
+@pytest.mark.parametrize("d,F,E,I,top,T", [(256, 64, 8, 4, 3, 21), (96, 40, 3, 0, 1, 21), (128, 200, 5, 2, 7, 21),
+                                            (256, 128, 6, 2, 3, 1), (128, 384, 3, 1, 2, 300), (384, 256, 9, 0, 4, 77)])
+def test_moe(dt, d, F, E, I, top, T):
+    """Widths on the 128 grid take the grouped MFMA GEMMs in bfloat16 (experts with no token, with one, with more
+    than a tile of them), every other case the token-parallel kernel."""
     from chronos.ops import hybrid as hops, hybrid_ref as ref
 
     g = _gen(d + F)
-    T = 21
     h = _rand(g, T, d, dtype=dt)
     wr = _rand(g, E + I, d, dtype=dt, scale=0.3)
     corr = _rand(g, E + I, scale=0.2)
