@@ -191,7 +191,7 @@ Tensor hy_latent_attention(const Tensor& qa, const Tensor& cache, const Tensor& 
         (int)B, (int)H, (int)DK, (int)rank, (int)cache.size(1), (int)std::max<int64_t>(1, max_q), (float)scale, f32(qa),
         stream());
     TORCH_CHECK(ok, "chronos hybrid op: latent_attention has no launch geometry for heads=", H, " row width=", DK,
-                " rank=", rank, " (heads <= 64, rank <= 512, one key tile and the query rows must fit the LDS)");
+                " rank=", rank, " (rank <= 512; 16 keys and 4 query rows must fit the LDS)");
     return out;
 }
 

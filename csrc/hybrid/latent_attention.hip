@@ -10,10 +10,12 @@
 //   latent_prep       per token: RMS norm of the latent columns (float), rotation of the shared key part and of
 //                     every head's rotated query columns (cos / sin from a float table made in double precision),
 //                     cache write at the token's page and slot.
-//   latent_attention  one workgroup per (sequence, tile of query tokens): the tile's (token, head) rows are split
+//   latent_attention  one workgroup per (sequence, block of up to 64 (token, head) rows): the rows are split
 //                     over 4 waves; 64-key tiles of the cache are staged in LDS; lanes are keys for the scores
 //                     (float accumulation, causal mask by each row's own position, online softmax in float) and
 //                     latent columns for the output.  Serves prefill chunks and decode rows (a tile of one token).
+#include <cstdlib>
+
 #include "hybrid_common.h"
 
 namespace chronos {
@@ -77,32 +79,35 @@ template <typename T, int DVL>
 __global__ void __launch_bounds__(256) latent_attention_kernel(
         const T* __restrict__ qa, const T* __restrict__ cache, const int32_t* __restrict__ block_table, int max_blocks,
         const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos, const float* __restrict__ gate,
-        T* __restrict__ out, int H, int DK, int rank, int BS, int QT, int KT, int kstride, float scale) {
+        T* __restrict__ out, int H, int DK, int rank, int BS, int RBLK, int KT, int kstride, float scale) {
     constexpr int E = Word<T>::E, RB = 4, RWMAX = 16;
     extern __shared__ __attribute__((aligned(16))) uint32_t smem[];
     const int b = blockIdx.x;
-    const int tq0 = q_start[b] + blockIdx.y * QT;
-    const int tq1 = min(tq0 + QT, q_start[b + 1]);
-    if (tq1 <= tq0) return;
-    const int ntok = tq1 - tq0, rows = ntok * H;
+    // rows of a sequence are (token * H + head); a workgroup takes RBLK (<= 64) consecutive rows, whatever H is
+    const int t0 = q_start[b];
+    const int rows_total = (q_start[b + 1] - t0) * H;
+    const int rb0 = blockIdx.y * RBLK;
+    if (rb0 >= rows_total) return;
+    const int rows = min(RBLK, rows_total - rb0);
     const int qwords = DK / E;
     uint32_t* ks = smem;
     uint32_t* qsm = ks + KT * kstride;
-    float* ps = reinterpret_cast<float*>(qsm + QT * H * qwords);
+    float* ps = reinterpret_cast<float*>(qsm + RBLK * qwords);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int rw = (rows + 3) / 4;          // rows per wave, <= RWMAX (host guarantees QT * H <= 64)
+    const int rw = (rows + 3) / 4;          // rows per wave, <= RWMAX (RBLK <= 64)
     const int r0 = wv * rw, r1 = min(rows, r0 + rw);
     // stage the tile's query rows (contiguous in qa)
-    const uint32_t* qg = reinterpret_cast<const uint32_t*>(qa + (int64_t)tq0 * H * DK);
+    const uint32_t* qg = reinterpret_cast<const uint32_t*>(qa + ((int64_t)t0 * H + rb0) * DK);
     for (int i = threadIdx.x; i < rows * qwords; i += 256) qsm[i] = qg[i];
-    const int pmax = pos[tq1 - 1];
+    const int pmax = pos[t0 + (rb0 + rows - 1) / H];
+    const bool vec16 = (qwords % 4) == 0;  // rows start 16-byte aligned then (the cache base is)
     float O[RWMAX][DVL], mrow[RWMAX], lrow[RWMAX];
     int prow[RWMAX];
 #pragma unroll
     for (int i = 0; i < RWMAX; ++i) {
         mrow[i] = -INFINITY;
         lrow[i] = 0.f;
-        prow[i] = (r0 + i < r1) ? pos[tq0 + (r0 + i) / H] : -1;
+        prow[i] = (r0 + i < r1) ? pos[t0 + (rb0 + r0 + i) / H] : -1;
 #pragma unroll
         for (int v = 0; v < DVL; ++v) O[i][v] = 0.f;
     }
@@ -111,11 +116,22 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     for (int k0 = 0; k0 <= pmax; k0 += KT) {
         __syncthreads();  // everyone is done with the previous key tile (and the query rows are staged)
         const int nk = min(KT, pmax + 1 - k0);
-        for (int i = threadIdx.x; i < nk * qwords; i += 256) {
-            const int j = i / qwords, wd = i % qwords;
+        // one wave per key row in turn (no index arithmetic per element; the page lookup is wave-uniform); 16-byte
+        // global loads where the row length allows, 4-byte LDS stores into the odd-stride rows
+        for (int j = wv; j < nk; j += 4) {
             const int key = k0 + j;
-            const uint32_t* src = reinterpret_cast<const uint32_t*>(cache + ((int64_t)bt[key / BS] * BS + key % BS) * DK);
-            ks[j * kstride + wd] = src[wd];
+            const T* rowp = cache + ((int64_t)bt[key / BS] * BS + key % BS) * DK;
+            uint32_t* dst = ks + j * kstride;
+            if (vec16) {
+                const uint4* src = reinterpret_cast<const uint4*>(rowp);
+                for (int p = lane; p < qwords / 4; p += 64) {
+                    const uint4 v = src[p];
+                    dst[4 * p] = v.x; dst[4 * p + 1] = v.y; dst[4 * p + 2] = v.z; dst[4 * p + 3] = v.w;
+                }
+            } else {
+                const uint32_t* src = reinterpret_cast<const uint32_t*>(rowp);
+                for (int p = lane; p < qwords; p += 64) dst[p] = src[p];
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -184,13 +200,13 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     for (int i = 0; i < RWMAX; ++i) {
         const int r = r0 + i;
         if (r < r1) {
-            const int tok = tq0 + r / H, hd = r % H;
+            const int64_t grow = (int64_t)t0 * H + rb0 + r;  // row of qa / gate / out
             float f = 1.f / lrow[i];
-            if (gate != nullptr) f *= sigmoidf_(gate[(int64_t)tok * H + hd]);
+            if (gate != nullptr) f *= sigmoidf_(gate[grow]);
 #pragma unroll
             for (int v = 0; v < DVL; ++v) {
                 const int col = lane + 64 * v;
-                if (col < rank) st<T>(out + ((int64_t)tok * H + hd) * rank + col, O[i][v] * f);
+                if (col < rank) st<T>(out + grow * rank + col, O[i][v] * f);
             }
         }
     }
@@ -206,23 +222,23 @@ void launch_hy_latent_prep(void* q, const void* dkv, const int32_t* pos, const i
     else hy::latent_prep_kernel<uint16_t><<<T, 256, 0, s>>>((uint16_t*)q, (const uint16_t*)dkv, pos, tok_seq, bt, max_blocks, w_norm, eps, cos_sin, dims, rank, R, H, D, (uint16_t*)cache, BS);
 }
 
-// Launch geometry of latent_attention for these sizes: QT query tokens per workgroup (QT * H <= 64 rows), KT keys per
+// Launch geometry of latent_attention for these sizes: RBLK (token, head) rows per workgroup (<= 64), KT keys per
 // LDS tile, the K tile's row stride in words (odd, so lanes reading consecutive rows hit different banks), and the
-// dynamic LDS bytes.  Returns false when no geometry fits the LDS (H > 64, or rows too wide).
-bool hy_latent_geometry(int H, int DK, int esize, int max_q, int lds_limit, int* QT, int* KT, int* kstride, int* bytes) {
-    if (H > 64 || H < 1) return false;
+// dynamic LDS bytes.  Returns false when not even 4 rows and 16 keys fit the LDS.
+bool hy_latent_geometry(int H, int DK, int esize, int max_q, int lds_limit, int* RBLK, int* KT, int* kstride, int* bytes) {
     const int qwords = DK * esize / 4;
-    int ks = qwords | 1;
-    int qt = 64 / H;
-    if (qt > max_q) qt = max_q < 1 ? 1 : max_q;
+    const int ks = qwords | 1;
+    int want = max_q * H;
+    if (want > 64) want = 64;
+    if (want < 1) want = 1;
     for (int kt = 64; kt >= 16; kt >>= 1) {
-        for (int q = qt; q >= 1; q = (q > 1 ? q / 2 : 0)) {
-            const int b = (kt * ks + q * H * qwords) * 4 + 4 * 64 * 4 * 4;
+        for (int r = want; r >= 4 || r == want; r = r / 2) {
+            const int b = (kt * ks + r * qwords) * 4 + 4 * 64 * 4 * 4;
             if (b <= lds_limit) {
-                *QT = q; *KT = kt; *kstride = ks; *bytes = b;
+                *RBLK = r; *KT = kt; *kstride = ks; *bytes = b;
                 return true;
             }
-            if (q == 1) break;
+            if (r <= 4) break;
         }
     }
     return false;
@@ -231,24 +247,36 @@ bool hy_latent_geometry(int H, int DK, int esize, int max_q, int lds_limit, int*
 template <typename T, int DVL>
 static void latent_attn_t(const T* qa, const T* cache, const int32_t* bt, int max_blocks, const int32_t* q_start,
                           const int32_t* pos, const float* gate, T* out, int B, int H, int DK, int rank, int BS,
-                          int max_q, int QT, int KT, int kstride, int bytes, float scale, hipStream_t s) {
+                          int max_q, int RBLK, int KT, int kstride, int bytes, float scale, hipStream_t s) {
     auto kern = hy::latent_attention_kernel<T, DVL>;
     static int set_bytes = 0;
     if (bytes > set_bytes) {  // raise the dynamic-LDS ceiling of this instantiation once per size
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         set_bytes = bytes;
     }
-    const dim3 grid(B, (max_q + QT - 1) / QT);
-    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, QT, KT, kstride, scale);
+    const dim3 grid(B, (max_q * H + RBLK - 1) / RBLK);
+    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, RBLK, KT, kstride, scale);
 }
+
+bool launch_hy_latent_attention_mfma(const uint16_t*, const uint16_t*, const int32_t*, int, const int32_t*, const int32_t*,
+                                     const float*, uint16_t*, int, int, int, int, int, int, float, hipStream_t);
 
 bool launch_hy_latent_attention(const void* qa, const void* cache, const int32_t* bt, int max_blocks,
                                 const int32_t* q_start, const int32_t* pos, const float* gate, void* out, int B, int H,
                                 int DK, int rank, int BS, int max_q, float scale, bool f32, hipStream_t s) {
     if (B == 0 || max_q == 0) return true;
-    int QT, KT, kstride, bytes;
-    if (rank > 512 || !hy_latent_geometry(H, DK, f32 ? 4 : 2, max_q, 160 * 1024, &QT, &KT, &kstride, &bytes)) return false;
-#define HY_LA(TT, DVL) latent_attn_t<TT, DVL>((const TT*)qa, (const TT*)cache, bt, max_blocks, q_start, pos, gate, (TT*)out, B, H, DK, rank, BS, max_q, QT, KT, kstride, bytes, scale, s)
+    // bfloat16 at MFMA-shaped sizes: the matrix-core kernel (CHRONOS_LATENT_MFMA=0 keeps the general one, for A/B)
+    static const bool use_mfma = [] {
+        const char* v = getenv("CHRONOS_LATENT_MFMA");
+        return v == nullptr || v[0] != '0';
+    }();
+    if (!f32 && use_mfma &&
+        launch_hy_latent_attention_mfma((const uint16_t*)qa, (const uint16_t*)cache, bt, max_blocks, q_start, pos, gate,
+                                        (uint16_t*)out, B, H, DK, rank, BS, max_q, scale, s))
+        return true;
+    int RBLK, KT, kstride, bytes;
+    if (rank > 512 || !hy_latent_geometry(H, DK, f32 ? 4 : 2, max_q, 160 * 1024, &RBLK, &KT, &kstride, &bytes)) return false;
+#define HY_LA(TT, DVL) latent_attn_t<TT, DVL>((const TT*)qa, (const TT*)cache, bt, max_blocks, q_start, pos, gate, (TT*)out, B, H, DK, rank, BS, max_q, RBLK, KT, kstride, bytes, scale, s)
     const int dvl = (rank + 63) / 64;
     if (f32) {
         if (dvl <= 1) HY_LA(float, 1); else if (dvl <= 2) HY_LA(float, 2); else if (dvl <= 4) HY_LA(float, 4); else HY_LA(float, 8);

@@ -1,0 +1,182 @@
+// latent_attention_mfma.hip — the bfloat16 latent attention on the matrix cores (see latent_attention.hip for the
+// math: one cached row per token, key = the whole row, value = its first `rank` columns, shared by all heads).
+//
+// One workgroup takes 64 (token, head) rows of one sequence — 16 per wave, rows are (token * H + head), so any head
+// count tiles the same way — and walks the sequence's keys 64 at a time:
+//   * the key tile is staged twice in LDS: row-major [64][DK] for the scores, and the value columns transposed
+//     [rank][64] for the weighted sum (both MFMA operands want 8 consecutive k-values per lane: dims for the scores,
+//     KEYS for the sum).  One pass of 16-byte global loads feeds both; the transposed image is written as 32-bit
+//     words holding two neighbouring keys.
+//   * scores  S^T = K Q^T : 16x16x32 MFMAs with the key rows as A operand and the wave's 16 query rows (held in
+//     registers for the whole kernel) as B operand, so a lane ends up with 4 keys x 1 query row per 16-key tile;
+//   * softmax in float per query row (lane & 15): causal mask by the row's own position, running maximum and sum,
+//     reductions over the 4 lane groups by two shuffles;
+//   * sum  O^T = V^T P^T : the lane's 8 weights of two neighbouring 16-key tiles ARE a B operand (the k index is a
+//     fixed permutation of the 32 keys, the same one the transposed value image is read with), so the weights never
+//     leave registers.  Accumulators: rank / 16 tiles x 4 registers.
+// Sizes: DK % 32 == 0, rank % 16 == 0, DK <= 576, rank <= 512.  Everything else takes latent_attention.hip.
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+constexpr int MKT = 64;  // keys per tile
+
+// NS: k-steps of the scores (DK / 32) at most; NCT: 16-column tiles of the output (rank / 16) at most.
+template <int NS, int NCT>
+__global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
+        const uint16_t* __restrict__ qa, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_table,
+        int max_blocks, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
+        const float* __restrict__ gate, uint16_t* __restrict__ out, int H, int DK, int rank, int BS, float scale) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int b = blockIdx.x;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    const int rows_total = (t1 - t0) * H;
+    const int rb0 = blockIdx.y * 64;
+    if (rb0 >= rows_total) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, g = lane >> 4, qi = lane & 15;
+    const int ns = DK / 32, nct = rank / 16;
+    const int krs = DK * 2 + 16;            // row-major image: bytes per key row
+    const int vts = MKT * 2 + 8;            // transposed image: bytes per value column
+    unsigned char* kimg = smem;
+    unsigned char* vimg = smem + MKT * krs;
+    // this lane's query row (for the B operand and for the softmax): row r of the sequence, token t0 + r / H
+    const int r = rb0 + wv * 16 + qi;
+    const bool rok = r < rows_total;
+    const int rc = rok ? r : rows_total - 1;
+    const int64_t grow = (int64_t)t0 * H + rc;              // row of qa / out / gate
+    const int prow = rok ? pos[t0 + rc / H] : -1;
+    const int last_row = min(rows_total, rb0 + 64) - 1;
+    const int pmax = pos[t0 + last_row / H];                // positions grow along the sequence
+    bf16x8 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        if (s < ns) qf[s] = *reinterpret_cast<const bf16x8*>(qa + grow * DK + 32 * s + 8 * g);
+    f32x4 O[NCT];
+#pragma unroll
+    for (int c = 0; c < NCT; ++c) O[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mrow = -INFINITY, lrow = 0.f;
+    const int32_t* bt = block_table + (int64_t)b * max_blocks;
+    const int chunks = DK / 8, vchunks = rank / 8;
+    for (int k0 = 0; k0 <= pmax; k0 += MKT) {
+        __syncthreads();
+        // ---- stage: work item = (key pair jp, 8-dim chunk dc); lanes of a wave take consecutive key pairs
+        for (int it = threadIdx.x; it < 32 * chunks; it += 256) {
+            const int jp = it & 31, dc = it >> 5;
+            const int ka = min(k0 + 2 * jp, pmax), kb = min(k0 + 2 * jp + 1, pmax);  // past the end: a real row, masked
+            const u16x8 va = *reinterpret_cast<const u16x8*>(cache + ((int64_t)bt[ka / BS] * BS + ka % BS) * DK + dc * 8);
+            const u16x8 vb = *reinterpret_cast<const u16x8*>(cache + ((int64_t)bt[kb / BS] * BS + kb % BS) * DK + dc * 8);
+            *reinterpret_cast<u16x8*>(kimg + (2 * jp) * krs + dc * 16) = va;
+            *reinterpret_cast<u16x8*>(kimg + (2 * jp + 1) * krs + dc * 16) = vb;
+            if (dc < vchunks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    *reinterpret_cast<uint32_t*>(vimg + (dc * 8 + e) * vts + jp * 4) = (uint32_t)va[e] | ((uint32_t)vb[e] << 16);
+            }
+        }
+        __syncthreads();
+        // ---- scores: 4 key tiles of 16; lane gets keys 16 kt + 4 g + i of query row qi
+        f32x4 S[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            S[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const unsigned char* arow = kimg + (16 * kt + qi) * krs + g * 16;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                if (s < ns)
+                    S[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(arow + s * 64), qf[s],
+                                                                    S[kt], 0, 0, 0);
+        }
+        // ---- softmax over the tile for query row qi (this lane and the 3 other lane groups hold its keys)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + 16 * kt + 4 * g + i;
+                const float sv = key <= prow ? S[kt][i] * scale : -INFINITY;
+                S[kt][i] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(mrow, mx);
+        const float corr = (mn == -INFINITY) ? 1.f : expf(mrow - mn);
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = (mn == -INFINITY) ? 0.f : expf(S[kt][i] - mn);
+                S[kt][i] = p;
+                sum += p;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        lrow = lrow * corr + sum;
+        mrow = mn;
+        // ---- weighted sum of the value columns: k index of step u = [tile 2u keys 4g..4g+3 | tile 2u+1 keys 4g..4g+3]
+        bf16x8 pf[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            pf[u] = bf16x8{(__bf16)S[2 * u][0], (__bf16)S[2 * u][1], (__bf16)S[2 * u][2], (__bf16)S[2 * u][3],
+                           (__bf16)S[2 * u + 1][0], (__bf16)S[2 * u + 1][1], (__bf16)S[2 * u + 1][2], (__bf16)S[2 * u + 1][3]};
+#pragma unroll
+        for (int c = 0; c < NCT; ++c) {
+            if (c < nct) {
+                O[c] *= corr;
+                const unsigned char* vrow = vimg + (16 * c + qi) * vts + g * 8;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow + u * 64);
+                    const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + u * 64 + 32);
+                    const bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    O[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], O[c], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!rok) return;
+    float f = 1.f / lrow;
+    if (gate != nullptr) f *= sigmoidf_(gate[grow]);
+    // lane holds O^T[col = 16 c + 4 g + i][query row qi]
+#pragma unroll
+    for (int c = 0; c < NCT; ++c)
+        if (c < nct) {
+            const u16x4 o = u16x4{f2bf(O[c][0] * f), f2bf(O[c][1] * f), f2bf(O[c][2] * f), f2bf(O[c][3] * f)};
+            *reinterpret_cast<u16x4*>(out + grow * rank + 16 * c + 4 * g) = o;
+        }
+}
+
+}  // namespace hy
+
+template <int NS, int NCT>
+static void la_mfma_launch(const uint16_t* qa, const uint16_t* cache, const int32_t* bt, int max_blocks,
+                           const int32_t* q_start, const int32_t* pos, const float* gate, uint16_t* out, int B, int H,
+                           int DK, int rank, int BS, int max_q, float scale, hipStream_t s) {
+    auto kern = hy::latent_attention_mfma_kernel<NS, NCT>;
+    const int bytes = hy::MKT * (DK * 2 + 16) + rank * (hy::MKT * 2 + 8);
+    static int set_bytes = 0;
+    if (bytes > set_bytes) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        set_bytes = bytes;
+    }
+    const dim3 grid(B, (max_q * H + 63) / 64);
+    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale);
+}
+
+// false: these sizes are not served here (the caller takes the general kernel)
+bool launch_hy_latent_attention_mfma(const uint16_t* qa, const uint16_t* cache, const int32_t* bt, int max_blocks,
+                                     const int32_t* q_start, const int32_t* pos, const float* gate, uint16_t* out, int B,
+                                     int H, int DK, int rank, int BS, int max_q, float scale, hipStream_t s) {
+    if (DK % 32 || rank % 16 || DK > 576 || rank > 512 || rank > DK) return false;
+    if (B == 0 || max_q == 0) return true;
+#define HY_LAM(NS, NCT) la_mfma_launch<NS, NCT>(qa, cache, bt, max_blocks, q_start, pos, gate, out, B, H, DK, rank, BS, max_q, scale, s)
+    if (DK <= 128 && rank <= 64) HY_LAM(4, 4);
+    else if (DK <= 320 && rank <= 256) HY_LAM(10, 16);
+    else HY_LAM(18, 32);
+#undef HY_LAM
+    return true;
+}
+
+}  // namespace chronos

@@ -131,7 +131,8 @@ def _paged(g, lens, starts, BS, DK, dt, shuffle=True):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,D,R,rank,dims", [(4, 32, 32, 64, 32), (3, 24, 16, 40, 8), (1, 8, 4, 130, 4), (8, 16, 64, 512, 64)])
+@pytest.mark.parametrize("H,D,R,rank,dims", [(4, 32, 32, 64, 32), (3, 24, 16, 40, 8), (1, 8, 4, 130, 4), (8, 16, 64, 512, 64),
+                                             (5, 16, 32, 160, 32), (1, 8, 16, 16, 16), (70, 8, 32, 96, 32)])
 def test_latent_prep_and_attention(dt, H, D, R, rank, dims):
     """Prefill portions over a cached prefix, decode rows, a first token; pages in shuffled order, partial last
     pages, query tiles that straddle key tiles."""
@@ -163,13 +164,14 @@ def test_latent_prep_and_attention(dt, H, D, R, rank, dims):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-def test_latent_attention_sees_exactly_its_prefix(dt):
+@pytest.mark.parametrize("R", [8, 32])
+def test_latent_attention_sees_exactly_its_prefix(dt, R):
     """One key far back carries a huge score and a marker value: a query at or after it must return the marker, the
     query just before it must not (causal edge, inside a prompt portion and for a decode row)."""
     from chronos.ops import hybrid as hops
 
     g = _gen(9)
-    H, rank, R, BS = 2, 32, 8, 16
+    H, rank, BS = 2, 32, 16     # (R = 32 in bfloat16: the matrix-core kernel; otherwise the general one)
     DK = rank + R
     lens, starts = [40, 1, 1], [100, 120, 119]
     q_start, _, pos, seq = _stream(lens, starts)
