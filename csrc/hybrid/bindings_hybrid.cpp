@@ -25,7 +25,10 @@ void launch_hy_mlstm_out(const float*, const void*, int, int, const float*, void
 void launch_hy_latent_prep(void*, const void*, const int32_t*, const int32_t*, const int32_t*, int, const float*, float,
                            const float*, int, int, int, int, int, void*, int, int, bool, hipStream_t);
 bool launch_hy_latent_attention(const void*, const void*, const int32_t*, int, const int32_t*, const int32_t*,
-                                const float*, void*, int, int, int, int, int, int, float, bool, hipStream_t);
+                                const float*, void*, int, int, int, int, int, int, float, bool, int, float*, float*, int64_t,
+                                hipStream_t);
+bool hy_latent_use_mfma(bool, int, int);
+int hy_latent_nsplit(int, int);
 void launch_hy_moe_route(const void*, const void*, const float*, int32_t*, float*, int, int, int, int, bool,
                          hipStream_t);
 void launch_hy_moe_ffn_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
@@ -185,11 +188,23 @@ Tensor hy_latent_attention(const Tensor& qa, const Tensor& cache, const Tensor& 
     if (gate) { flt(*gate, "latent_attention: float32 gate"); need(gate->numel() == T * H, "latent_attention: gate [T, H]"); }
     auto out = at::empty({T, H, rank}, qa.options());
     if (T == 0 || B <= 0) return out;
+    // few workgroups over long contexts (decode rows, a lone short portion): split the key range over more workgroups
+    // and merge the partials; the split count follows from sizes the host knows (the block table bounds the context)
+    const int mq = (int)std::max<int64_t>(1, max_q);
+    int nsplit = 1;
+    Tensor part_o, part_ml;
+    if (chronos::hy_latent_use_mfma(f32(qa), (int)DK, (int)rank)) {
+        nsplit = chronos::hy_latent_nsplit((int)(B * ((mq * H + 63) / 64)), (int)(block_table.size(1) * cache.size(1)));
+        if (nsplit > 1) {
+            part_o = at::empty({T * H * nsplit, rank}, qa.options().dtype(at::kFloat));
+            part_ml = at::empty({T * H * nsplit, 2}, qa.options().dtype(at::kFloat));
+        }
+    }
     const bool ok = chronos::launch_hy_latent_attention(
         qa.data_ptr(), cache.data_ptr(), block_table.data_ptr<int32_t>(), (int)block_table.size(1),
         q_start.data_ptr<int32_t>(), pos.data_ptr<int32_t>(), gate ? gate->data_ptr<float>() : nullptr, out.data_ptr(),
-        (int)B, (int)H, (int)DK, (int)rank, (int)cache.size(1), (int)std::max<int64_t>(1, max_q), (float)scale, f32(qa),
-        stream());
+        (int)B, (int)H, (int)DK, (int)rank, (int)cache.size(1), mq, (float)scale, f32(qa), nsplit,
+        nsplit > 1 ? part_o.data_ptr<float>() : nullptr, nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, T * H, stream());
     TORCH_CHECK(ok, "chronos hybrid op: latent_attention has no launch geometry for heads=", H, " row width=", DK,
                 " rank=", rank, " (rank <= 512; 16 keys and 4 query rows must fit the LDS)");
     return out;

@@ -259,21 +259,29 @@ static void latent_attn_t(const T* qa, const T* cache, const int32_t* bt, int ma
 }
 
 bool launch_hy_latent_attention_mfma(const uint16_t*, const uint16_t*, const int32_t*, int, const int32_t*, const int32_t*,
-                                     const float*, uint16_t*, int, int, int, int, int, int, float, hipStream_t);
+                                     const float*, uint16_t*, int, int, int, int, int, int, float, int, float*, float*,
+                                     int64_t, hipStream_t);
+bool hy_latent_mfma_ok(int DK, int rank);
 
-bool launch_hy_latent_attention(const void* qa, const void* cache, const int32_t* bt, int max_blocks,
-                                const int32_t* q_start, const int32_t* pos, const float* gate, void* out, int B, int H,
-                                int DK, int rank, int BS, int max_q, float scale, bool f32, hipStream_t s) {
-    if (B == 0 || max_q == 0) return true;
-    // bfloat16 at MFMA-shaped sizes: the matrix-core kernel (CHRONOS_LATENT_MFMA=0 keeps the general one, for A/B)
-    static const bool use_mfma = [] {
+// whether this call goes to the matrix-core kernel (bfloat16 at its sizes; CHRONOS_LATENT_MFMA=0 keeps the general
+// kernel, for A/B)
+bool hy_latent_use_mfma(bool f32, int DK, int rank) {
+    static const bool on = [] {
         const char* v = getenv("CHRONOS_LATENT_MFMA");
         return v == nullptr || v[0] != '0';
     }();
-    if (!f32 && use_mfma &&
-        launch_hy_latent_attention_mfma((const uint16_t*)qa, (const uint16_t*)cache, bt, max_blocks, q_start, pos, gate,
-                                        (uint16_t*)out, B, H, DK, rank, BS, max_q, scale, s))
-        return true;
+    return !f32 && on && hy_latent_mfma_ok(DK, rank);
+}
+
+bool launch_hy_latent_attention(const void* qa, const void* cache, const int32_t* bt, int max_blocks,
+                                const int32_t* q_start, const int32_t* pos, const float* gate, void* out, int B, int H,
+                                int DK, int rank, int BS, int max_q, float scale, bool f32, int nsplit, float* part_o,
+                                float* part_ml, int64_t total_rows, hipStream_t s) {
+    if (B == 0 || max_q == 0) return true;
+    if (hy_latent_use_mfma(f32, DK, rank))
+        return launch_hy_latent_attention_mfma((const uint16_t*)qa, (const uint16_t*)cache, bt, max_blocks, q_start, pos, gate,
+                                               (uint16_t*)out, B, H, DK, rank, BS, max_q, scale, nsplit, part_o, part_ml,
+                                               total_rows, s);
     int RBLK, KT, kstride, bytes;
     if (rank > 512 || !hy_latent_geometry(H, DK, f32 ? 4 : 2, max_q, 160 * 1024, &RBLK, &KT, &kstride, &bytes)) return false;
 #define HY_LA(TT, DVL) latent_attn_t<TT, DVL>((const TT*)qa, (const TT*)cache, bt, max_blocks, q_start, pos, gate, (TT*)out, B, H, DK, rank, BS, max_q, RBLK, KT, kstride, bytes, scale, s)

@@ -27,7 +27,8 @@ template <int NS, int NCT>
 __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         const uint16_t* __restrict__ qa, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_table,
         int max_blocks, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
-        const float* __restrict__ gate, uint16_t* __restrict__ out, int H, int DK, int rank, int BS, float scale) {
+        const float* __restrict__ gate, uint16_t* __restrict__ out, int H, int DK, int rank, int BS, float scale,
+        int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int b = blockIdx.x;
     const int t0 = q_start[b], t1 = q_start[b + 1];
@@ -58,7 +59,9 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     float mrow = -INFINITY, lrow = 0.f;
     const int32_t* bt = block_table + (int64_t)b * max_blocks;
     const int chunks = DK / 8, vchunks = rank / 8;
-    for (int k0 = 0; k0 <= pmax; k0 += MKT) {
+    // key tiles are dealt round-robin to the nsplit workgroups of this row block (blockIdx.z): the context length is
+    // only known on the device, and a split that gets no tile contributes an empty partial
+    for (int k0 = blockIdx.z * MKT; k0 <= pmax; k0 += MKT * nsplit) {
         __syncthreads();
         // ---- stage: work item = (key pair jp, 8-dim chunk dc); lanes of a wave take consecutive key pairs
         for (int it = threadIdx.x; it < 32 * chunks; it += 256) {
@@ -137,6 +140,17 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         }
     }
     if (!rok) return;
+    if (nsplit > 1) {  // unnormalised partial: the combine kernel merges the splits
+        const int64_t pr = grow * nsplit + blockIdx.z;
+        if (g == 0) {
+            part_ml[pr * 2] = mrow;
+            part_ml[pr * 2 + 1] = lrow;
+        }
+#pragma unroll
+        for (int c = 0; c < NCT; ++c)
+            if (c < nct) *reinterpret_cast<f32x4*>(part_o + pr * rank + 16 * c + 4 * g) = O[c];
+        return;
+    }
     float f = 1.f / lrow;
     if (gate != nullptr) f *= sigmoidf_(gate[grow]);
     // lane holds O^T[col = 16 c + 4 g + i][query row qi]
@@ -148,12 +162,39 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         }
 }
 
+// one wave per (token, head) row: out = sum_z exp(m_z - m) O_z / sum_z exp(m_z - m) l_z * sigmoid(gate)
+__global__ void __launch_bounds__(256) latent_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                             const float* __restrict__ gate, uint16_t* __restrict__ out,
+                                                             int64_t rows, int rank, int nsplit) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    float m = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) m = fmaxf(m, part_ml[(r * nsplit + z) * 2]);
+    float l = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+        const float mz = part_ml[(r * nsplit + z) * 2];
+        if (mz != -INFINITY) l += expf(mz - m) * part_ml[(r * nsplit + z) * 2 + 1];
+    }
+    float f = 1.f / l;
+    if (gate != nullptr) f *= sigmoidf_(gate[r]);
+    for (int c = lane; c < rank; c += 64) {
+        float acc = 0.f;
+        for (int z = 0; z < nsplit; ++z) {
+            const float mz = part_ml[(r * nsplit + z) * 2];
+            if (mz != -INFINITY) acc += expf(mz - m) * part_o[(r * nsplit + z) * rank + c];
+        }
+        out[r * rank + c] = f2bf(acc * f);
+    }
+}
+
 }  // namespace hy
 
 template <int NS, int NCT>
 static void la_mfma_launch(const uint16_t* qa, const uint16_t* cache, const int32_t* bt, int max_blocks,
                            const int32_t* q_start, const int32_t* pos, const float* gate, uint16_t* out, int B, int H,
-                           int DK, int rank, int BS, int max_q, float scale, hipStream_t s) {
+                           int DK, int rank, int BS, int max_q, float scale, int nsplit, float* part_o, float* part_ml,
+                           hipStream_t s) {
     auto kern = hy::latent_attention_mfma_kernel<NS, NCT>;
     const int bytes = hy::MKT * (DK * 2 + 16) + rank * (hy::MKT * 2 + 8);
     static int set_bytes = 0;
@@ -161,21 +202,38 @@ static void la_mfma_launch(const uint16_t* qa, const uint16_t* cache, const int3
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         set_bytes = bytes;
     }
-    const dim3 grid(B, (max_q * H + 63) / 64);
-    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale);
+    const dim3 grid(B, (max_q * H + 63) / 64, nsplit);
+    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale, nsplit, part_o,
+                                  part_ml);
 }
 
-// false: these sizes are not served here (the caller takes the general kernel)
+bool hy_latent_mfma_ok(int DK, int rank) { return !(DK % 32 || rank % 16 || DK > 576 || rank > 512 || rank > DK); }
+
+// Splits of the key range (flash-decoding) for a launch of `wgs` workgroups over contexts of at most max_ctx keys:
+// enough workgroups to cover the chip, at least 4 key tiles per split, at most 16.
+int hy_latent_nsplit(int wgs, int max_ctx) {
+    if (wgs >= 128) return 1;
+    int want = (256 + wgs - 1) / wgs, cap = max_ctx / (4 * hy::MKT);
+    if (want > 16) want = 16;
+    if (want > cap) want = cap;
+    return want < 1 ? 1 : want;
+}
+
+// false: these sizes are not served here (the caller takes the general kernel).  nsplit > 1: part_o float
+// [T * H * nsplit, rank] and part_ml float [T * H * nsplit, 2] scratch.
 bool launch_hy_latent_attention_mfma(const uint16_t* qa, const uint16_t* cache, const int32_t* bt, int max_blocks,
                                      const int32_t* q_start, const int32_t* pos, const float* gate, uint16_t* out, int B,
-                                     int H, int DK, int rank, int BS, int max_q, float scale, hipStream_t s) {
-    if (DK % 32 || rank % 16 || DK > 576 || rank > 512 || rank > DK) return false;
+                                     int H, int DK, int rank, int BS, int max_q, float scale, int nsplit, float* part_o,
+                                     float* part_ml, int64_t total_rows, hipStream_t s) {
+    if (!hy_latent_mfma_ok(DK, rank)) return false;
     if (B == 0 || max_q == 0) return true;
-#define HY_LAM(NS, NCT) la_mfma_launch<NS, NCT>(qa, cache, bt, max_blocks, q_start, pos, gate, out, B, H, DK, rank, BS, max_q, scale, s)
+#define HY_LAM(NS, NCT) la_mfma_launch<NS, NCT>(qa, cache, bt, max_blocks, q_start, pos, gate, out, B, H, DK, rank, BS, max_q, scale, nsplit, part_o, part_ml, s)
     if (DK <= 128 && rank <= 64) HY_LAM(4, 4);
     else if (DK <= 320 && rank <= 256) HY_LAM(10, 16);
     else HY_LAM(18, 32);
 #undef HY_LAM
+    if (nsplit > 1)
+        hy::latent_combine_kernel<<<(unsigned)((total_rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, gate, out, total_rows, rank, nsplit);
     return true;
 }
 

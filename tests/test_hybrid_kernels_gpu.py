@@ -213,3 +213,25 @@ def test_moe(dt, d, F, E, I, top, T):
         y = hops.moe_ffn(h, idx2, wt2, wu, wd, act, dt)
         y2 = ref.moe_ffn(h, idx2, wt2, wu, wd, act, dt)
         _close(y, y2, _tol(dt, 2e-5, 1.5e-2))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("H,R,rank", [(4, 32, 64), (16, 64, 512), (3, 8, 40)])
+def test_latent_attention_long_context_few_rows(dt, H, R, rank):
+    """Decode rows and a two-token portion over contexts of very different lengths (3 to 1500 keys) behind a wide
+    block table: the bfloat16 matrix-core kernel splits the key range over several workgroups and merges the
+    partials; splits that get no key tile must not disturb the result."""
+    from chronos.ops import hybrid as hops, hybrid_ref as ref
+
+    g = _gen(H + rank)
+    BS, DK = 16, rank + R
+    lens, starts = [1, 1, 2, 1], [1499, 700, 2, 255]
+    q_start, _, pos, _ = _stream(lens, starts)
+    cache, bt = _paged(g, lens, starts, BS, DK, dt)
+    wide = torch.zeros(len(lens), 128, dtype=torch.int32, device=DEV)
+    wide[:, :bt.shape[1]] = bt
+    qa = _rand(g, sum(lens), H, DK, dtype=dt, scale=0.3)
+    gate = _rand(g, sum(lens), H)
+    o = hops.latent_attention(qa, cache, wide, q_start, pos, gate, 0.2, rank, dt, max(lens))
+    o2 = ref.latent_attention(qa, cache, wide, q_start, pos, gate, 0.2, rank, dt)
+    _close(o, o2, _tol(dt, 2e-5, 1e-2))
