@@ -29,7 +29,7 @@ bool launch_hy_latent_attention(const void*, const void*, const int32_t*, int, c
                                 hipStream_t);
 bool hy_latent_use_mfma(bool, int, int);
 int hy_latent_nsplit(int, int);
-void launch_hy_moe_route(const void*, const void*, const float*, int32_t*, float*, int, int, int, int, bool,
+void launch_hy_moe_route(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
                          hipStream_t);
 void launch_hy_moe_ffn_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
                              int, int, int, bool, hipStream_t);
@@ -219,7 +219,8 @@ std::tuple<Tensor, Tensor> hy_moe_route(const Tensor& h, const Tensor& w, const 
     need(corr.numel() == N && N <= 256 && top >= 1 && top <= N, "moe_route: 1 <= top <= outputs <= 256");
     auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
     auto wt = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
-    chronos::launch_hy_moe_route(h.data_ptr(), w.data_ptr(), corr.data_ptr<float>(), idx.data_ptr<int32_t>(),
+    auto z = at::empty({h.size(0), N}, h.options().dtype(at::kFloat));
+    chronos::launch_hy_moe_route(h.data_ptr(), w.data_ptr(), corr.data_ptr<float>(), z.data_ptr<float>(), idx.data_ptr<int32_t>(),
                                  wt.data_ptr<float>(), (int)h.size(0), (int)h.size(1), (int)N, (int)top, f32(h), stream());
     return {idx, wt};
 }

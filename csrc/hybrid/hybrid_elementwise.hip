@@ -57,20 +57,36 @@ __global__ void __launch_bounds__(256) layer_norm_kernel(const TY* __restrict__ 
     }
 }
 
-// out[t, n] = sum_k h[t, k] * w[n, k] (+ bias[n]) in float: one workgroup per token, one wave per output row in turn.
-template <typename T>
+// out[t, n] = sum_k h[t, k] * w[n, k] (+ bias[n]) in float.  One workgroup per TB tokens, whose rows sit in LDS; a
+// wave takes the output rows in turn and reads each weight row ONCE for all TB tokens (the weights are re-read per
+// workgroup from L2, so tokens per workgroup divide that traffic).
+template <typename T, int TB>
 __global__ void __launch_bounds__(256) rowdot_kernel(const T* __restrict__ h, const T* __restrict__ w,
-                                                     const float* __restrict__ bias, float* __restrict__ out, int d,
-                                                     int n) {
-    const int64_t t = blockIdx.x;
+                                                     const float* __restrict__ bias, float* __restrict__ out, int rows,
+                                                     int d, int n) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char rd_smem[];
+    T* hs = reinterpret_cast<T*>(rd_smem);
+    const int64_t t0 = (int64_t)blockIdx.x * TB;
+    const int nt = (int)min((int64_t)TB, rows - t0);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const T* hr = h + t * d;
+    for (int i = threadIdx.x; i < nt * d; i += 256) hs[i] = h[t0 * d + i];
+    __syncthreads();
     for (int r = wv; r < n; r += 4) {
         const T* wr = w + (int64_t)r * d;
-        float acc = 0.f;
-        for (int k = lane; k < d; k += 64) acc += ld<T>(hr + k) * ld<T>(wr + k);
-        acc = wave_sum(acc);
-        if (lane == 0) out[t * n + r] = acc + (bias != nullptr ? bias[r] : 0.f);
+        float acc[TB];
+#pragma unroll
+        for (int u = 0; u < TB; ++u) acc[u] = 0.f;
+        for (int k = lane; k < d; k += 64) {
+            const float wk = ld<T>(wr + k);
+#pragma unroll
+            for (int u = 0; u < TB; ++u)
+                if (u < nt) acc[u] += ld<T>(hs + u * d + k) * wk;
+        }
+#pragma unroll
+        for (int u = 0; u < TB; ++u) {
+            const float v = wave_sum(acc[u]);
+            if (lane == 0 && u < nt) out[(t0 + u) * n + r] = v + (bias != nullptr ? bias[r] : 0.f);
+        }
     }
 }
 
@@ -104,11 +120,30 @@ void launch_hy_layer_norm(const void* y, bool y_f32, float* x, const float* w, v
         else hy::layer_norm_kernel<float, uint16_t, false><<<rows, 256, 0, s>>>((const float*)y, nullptr, w, (uint16_t*)h, d, eps);
     }
 }
+template <typename T>
+static void rowdot_t(const T* h, const T* w, const float* bias, float* out, int rows, int d, int n, hipStream_t s) {
+    // tokens per workgroup: as many (up to 8) as keep the staged rows within 48 KB
+    const int fit = (48 * 1024) / (d * (int)sizeof(T));
+#define HY_RD(TB)                                                                                              \
+    hy::rowdot_kernel<T, TB><<<(rows + TB - 1) / TB, 256, TB * d * sizeof(T), s>>>(h, w, bias, out, rows, d, n)
+    if (fit >= 8 && rows >= 8) HY_RD(8);
+    else if (fit >= 4 && rows >= 4) HY_RD(4);
+    else if (fit >= 2 && rows >= 2) HY_RD(2);
+    else {
+        auto kern = hy::rowdot_kernel<T, 1>;
+        const int bytes = d * (int)sizeof(T);
+        if (bytes > 48 * 1024)
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<rows, 256, bytes, s>>>(h, w, bias, out, rows, d, n);
+    }
+#undef HY_RD
+}
+
 void launch_hy_rowdot(const void* h, const void* w, const float* bias, float* out, int T, int d, int n, bool f32,
                       hipStream_t s) {
     if (T == 0 || n == 0) return;
-    if (f32) hy::rowdot_kernel<float><<<T, 256, 0, s>>>((const float*)h, (const float*)w, bias, out, d, n);
-    else hy::rowdot_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)h, (const uint16_t*)w, bias, out, d, n);
+    if (f32) rowdot_t<float>((const float*)h, (const float*)w, bias, out, T, d, n, s);
+    else rowdot_t<uint16_t>((const uint16_t*)h, (const uint16_t*)w, bias, out, T, d, n, s);
 }
 void launch_hy_act(void* x, int64_t n, int kind, bool f32, hipStream_t s) {
     if (n == 0) return;

@@ -22,13 +22,27 @@
 namespace chronos {
 namespace hy {
 
+// Tokens are taken TG at a time (TG <= 64, a power of two): lane t evaluates the gates of token t (the tanh / log /
+// exp work runs across the lanes, not along the sequence), the running maximum is a short scalar recurrence over the
+// block, and the block's k and q rows are staged in LDS with coalesced loads, so the sequential n update never waits
+// on global memory.  LDS: k rows [TG][D] | q rows [TG][D] in the activation type, then 5 float arrays of 64.
 template <typename T>
-__global__ void __launch_bounds__(64) mlstm_gate_scan_kernel(
+__global__ void __launch_bounds__(256) mlstm_gate_scan_kernel(
         const T* __restrict__ proj, int ldp, const float* __restrict__ gate_pre, const int32_t* __restrict__ q_start,
         const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots, float* __restrict__ n_state,
         float* __restrict__ m_state, float* __restrict__ a_out, float* __restrict__ b_out, float* __restrict__ den_out,
-        int H, int D, float cap) {
-    const int b = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x;
+        int H, int D, float cap, int TG, int vec) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char gs_smem[];
+    T* kst = reinterpret_cast<T*>(gs_smem);
+    T* qst = kst + (size_t)TG * D;
+    float* ig_s = reinterpret_cast<float*>(qst + (size_t)TG * D);
+    float* fg_s = ig_s + 64;
+    float* a_s = fg_s + 64;
+    float* b_s = a_s + 64;
+    float* em_s = b_s + 64;
+    // 256 threads stage the block's rows (16-byte loads, 8 in flight per thread); wave 0 runs the recurrences
+    const int b = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63;
+    const bool w0 = threadIdx.x < 64;
     const int t0 = q_start[b], t1 = q_start[b + 1];
     if (t1 <= t0) return;
     const int slot = slots[b];
@@ -43,37 +57,92 @@ __global__ void __launch_bounds__(64) mlstm_gate_scan_kernel(
     }
     float m = fresh ? 0.f : m_state[(int64_t)slot * H + hd];
     const float qs = 1.f / sqrtf((float)D);
-    for (int t = t0; t < t1; ++t) {
-        const float zi = gate_pre[(int64_t)t * 2 * H + hd], zf = gate_pre[(int64_t)t * 2 * H + H + hd];
-        const float ig = cap * tanhf(zi / cap);
-        const float fg = logsigmoidf_(cap * tanhf(zf / cap));
-        const float mn = fmaxf(fg + m, ig);
-        const float a = expf(fg + m - mn), bb = expf(ig - mn);
-        m = mn;
-        const T* q = proj + (int64_t)t * ldp + hd * D;
-        const T* k = proj + (int64_t)t * ldp + H * D + hd * D;
-        float dot = 0.f;
+    for (int tb = t0; tb < t1; tb += TG) {
+        const int nt = min(TG, t1 - tb);
+        __syncthreads();  // the previous block's rows are no longer read
+        if (w0 && lane < nt) {
+            const float zi = gate_pre[(int64_t)(tb + lane) * 2 * H + hd], zf = gate_pre[(int64_t)(tb + lane) * 2 * H + H + hd];
+            ig_s[lane] = cap * tanhf(zi / cap);
+            fg_s[lane] = logsigmoidf_(cap * tanhf(zf / cap));
+        }
+        if (vec) {
+            constexpr int EV = 16 / (int)sizeof(T);
+            const int vpr = D / EV, nvec = nt * 2 * vpr;  // vectors per row; per token: q row | k row
+            for (int base = threadIdx.x; base < nvec; base += 256 * 8) {
+                uint4 r[8];
 #pragma unroll
-        for (int j = 0; j < NL; ++j) {
-            const int dd = lane + 64 * j;
-            if (dd < D) {
-                n[j] = a * n[j] + bb * ld<T>(k + dd);
-                dot += n[j] * (ld<T>(q + dd) * qs);
+                for (int u = 0; u < 8; ++u) {
+                    const int v = base + 256 * u;
+                    if (v < nvec) {
+                        const int tt = v / (2 * vpr), rem = v - tt * 2 * vpr;
+                        const int part = rem >= vpr, off = (rem - part * vpr) * EV;
+                        r[u] = *reinterpret_cast<const uint4*>(proj + (int64_t)(tb + tt) * ldp + (part ? H * D : 0) + hd * D + off);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int v = base + 256 * u;
+                    if (v < nvec) {
+                        const int tt = v / (2 * vpr), rem = v - tt * 2 * vpr;
+                        const int part = rem >= vpr, off = (rem - part * vpr) * EV;
+                        *reinterpret_cast<uint4*>((part ? kst : qst) + tt * D + off) = r[u];
+                    }
+                }
+            }
+        } else {
+            for (int tt = 0; tt < nt; ++tt) {
+                const T* row = proj + (int64_t)(tb + tt) * ldp + hd * D;
+                for (int dd = threadIdx.x; dd < D; dd += 256) {
+                    qst[tt * D + dd] = row[dd];
+                    kst[tt * D + dd] = row[(int64_t)H * D + dd];
+                }
             }
         }
-        dot = wave_sum(dot);
-        if (lane == 0) {
-            a_out[(int64_t)t * H + hd] = a;
-            b_out[(int64_t)t * H + hd] = bb;
-            den_out[(int64_t)t * H + hd] = fmaxf(fabsf(dot), expf(-m)) + 1e-6f;
+        __syncthreads();
+        if (!w0) continue;  // (the loop's first barrier keeps these waves in step)
+        // running maximum: every lane walks the block, lane t keeps (m_{t-1}, m_t)
+        float mp = m, mine_prev = m, mine = m;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float mn = fmaxf(fg_s[tt] + mp, ig_s[tt]);
+            if (tt == lane) {
+                mine_prev = mp;
+                mine = mn;
+            }
+            mp = mn;
         }
+        m = mp;
+        if (lane < nt) {
+            const float a = expf(fg_s[lane] + mine_prev - mine), bb = expf(ig_s[lane] - mine);
+            a_s[lane] = a;
+            b_s[lane] = bb;
+            em_s[lane] = expf(-mine);
+            a_out[(int64_t)(tb + lane) * H + hd] = a;
+            b_out[(int64_t)(tb + lane) * H + hd] = bb;
+        }
+        __builtin_amdgcn_wave_barrier();  // wave 0's own LDS writes above, read by its lanes below
+        float den_mine = 0.f;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float a = a_s[tt], bb = b_s[tt];
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < NL; ++j) {
+                const int dd = lane + 64 * j;
+                if (dd < D) {
+                    n[j] = a * n[j] + bb * ld<T>(kst + tt * D + dd);
+                    dot += n[j] * (ld<T>(qst + tt * D + dd) * qs);
+                }
+            }
+            dot = wave_sum(dot);
+            if (tt == lane) den_mine = fmaxf(fabsf(dot), em_s[tt]) + 1e-6f;
+        }
+        if (lane < nt) den_out[(int64_t)(tb + lane) * H + hd] = den_mine;
     }
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
         const int dd = lane + 64 * j;
-        if (dd < D) ns[dd] = n[j];
+        if (w0 && dd < D) ns[dd] = n[j];
     }
-    if (lane == 0) m_state[(int64_t)slot * H + hd] = m;
+    if (threadIdx.x == 0) m_state[(int64_t)slot * H + hd] = m;
 }
 
 // DR: state rows per wave (D <= 4 * DR).  TT tokens per LDS stage.
@@ -156,6 +225,122 @@ __global__ void __launch_bounds__(256) mlstm_state_scan_kernel(
     }
 }
 
+// The same scan with 16-byte global loads and the NEXT stage's loads in flight while the current stage's tokens are
+// processed (the sequential token loop leaves one workgroup per CU alone with its memory latency otherwise).
+// Needs rows of q, k, v that start and end on 16-byte boundaries (host-checked).  TT = 16 tokens per stage.
+template <typename T, int DR>
+__global__ void __launch_bounds__(256) mlstm_state_scan_vec_kernel(
+        const T* __restrict__ proj, int ldp, const float* __restrict__ a_in, const float* __restrict__ b_in,
+        const float* __restrict__ den_in, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0,
+        const int32_t* __restrict__ slots, float* __restrict__ S_state, float* __restrict__ o_out, int H, int D,
+        int Dv) {
+    constexpr int TT = 16, DP = 4 * DR, EV = 16 / (int)sizeof(T);     // elements per 16-byte vector
+    constexpr int QV = DP / EV, VV = 64 / EV, PV = 2 * QV + VV;       // vectors per token: q | k | v slice
+    constexpr int NV = (TT * PV + 255) / 256;                         // vectors per thread and stage
+    __shared__ __attribute__((aligned(16))) float qs_[TT][DP];
+    __shared__ __attribute__((aligned(16))) float ks_[TT][DP];
+    __shared__ __attribute__((aligned(16))) float vs_[TT][64];
+    __shared__ float ab_[TT][2];
+    __shared__ float part_[4][TT][64];
+    const int b = blockIdx.x, hd = blockIdx.y, c0 = blockIdx.z * 64;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    if (t1 <= t0) return;
+    const int slot = slots[b];
+    const bool fresh = pos0[b] == 0;
+    const int c = c0 + lane;
+    const bool cok = c < Dv;
+    float* Ss = S_state + (((int64_t)slot * H + hd) * D) * Dv;
+    const int d0 = wv * DR;
+    float S[DR];
+#pragma unroll
+    for (int j = 0; j < DR; ++j) S[j] = (!fresh && cok && d0 + j < D) ? Ss[(int64_t)(d0 + j) * Dv + c] : 0.f;
+    const float qscale = 1.f / sqrtf((float)D);
+    const int qoff = hd * D, koff = H * D + hd * D, voff = 2 * H * D + hd * Dv + c0;
+    uint4 raw[NV];
+    auto fetch = [&](int tb) {
+        const int nt = min(TT, t1 - tb);
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int v = threadIdx.x + 256 * u;
+            const int tt = v / PV, rem = v % PV;
+            const int part = rem < QV ? 0 : (rem < 2 * QV ? 1 : 2);
+            const int e = (part == 0 ? rem : (part == 1 ? rem - QV : rem - 2 * QV)) * EV;
+            const bool ok = tt < nt && (part == 2 ? c0 + e < Dv : e < D);
+            const T* src = proj + (int64_t)(tb + tt) * ldp + (part == 0 ? qoff : (part == 1 ? koff : voff)) + e;
+            raw[u] = ok ? *reinterpret_cast<const uint4*>(src) : uint4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto store = [&]() {
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int v = threadIdx.x + 256 * u;
+            const int tt = v / PV, rem = v % PV;
+            if (tt >= TT) continue;
+            const int part = rem < QV ? 0 : (rem < 2 * QV ? 1 : 2);
+            const int e = (part == 0 ? rem : (part == 1 ? rem - QV : rem - 2 * QV)) * EV;
+            float* dst = part == 0 ? &qs_[tt][e] : (part == 1 ? &ks_[tt][e] : &vs_[tt][e]);
+            const float sc = part == 0 ? qscale : 1.f;
+            float f[EV];
+            if constexpr (sizeof(T) == 2) {
+                const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    f[2 * i] = __uint_as_float(w[i] << 16) * sc;
+                    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * sc;
+                }
+            } else {
+                f[0] = __uint_as_float(raw[u].x) * sc; f[1] = __uint_as_float(raw[u].y) * sc;
+                f[2] = __uint_as_float(raw[u].z) * sc; f[3] = __uint_as_float(raw[u].w) * sc;
+            }
+#pragma unroll
+            for (int i = 0; i < EV; i += 4) *reinterpret_cast<f32x4*>(dst + i) = f32x4{f[i], f[i + 1], f[i + 2], f[i + 3]};
+        }
+    };
+    fetch(t0);
+    for (int tb = t0; tb < t1; tb += TT) {
+        const int nt = min(TT, t1 - tb);
+        __syncthreads();  // the previous stage's LDS is no longer read
+        store();
+        if (threadIdx.x < TT * 2) {
+            const int tt = threadIdx.x >> 1, which = threadIdx.x & 1;
+            float v = which ? 0.f : 1.f;
+            if (tt < nt) v = (which ? b_in : a_in)[(int64_t)(tb + tt) * H + hd];
+            ab_[tt][which] = v;
+        }
+        if (tb + TT < t1) fetch(tb + TT);  // in flight during this stage's token loop
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float a = ab_[tt][0], bv = ab_[tt][1] * vs_[tt][lane];
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < DR; j += 4) {
+                const f32x4 kk = *reinterpret_cast<const f32x4*>(&ks_[tt][d0 + j]);
+                const f32x4 qq = *reinterpret_cast<const f32x4*>(&qs_[tt][d0 + j]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    S[j + u] = a * S[j + u] + kk[u] * bv;
+                    acc += S[j + u] * qq[u];
+                }
+            }
+            part_[wv][tt][lane] = acc;
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < nt * 64; i += 256) {
+            const int tt = i >> 6, l = i & 63;
+            if (c0 + l < Dv) {
+                const float num = (part_[0][tt][l] + part_[1][tt][l]) + (part_[2][tt][l] + part_[3][tt][l]);
+                o_out[((int64_t)(tb + tt) * H + hd) * Dv + c0 + l] = num / den_in[(int64_t)(tb + tt) * H + hd];
+            }
+        }
+    }
+    if (cok) {
+#pragma unroll
+        for (int j = 0; j < DR; ++j)
+            if (d0 + j < D) Ss[(int64_t)(d0 + j) * Dv + c] = S[j];
+    }
+}
+
 // one wave per (token, head): y = o * rsqrt(mean(o^2) + eps) * w[head, :] * sigmoid(g[token, head, :])
 template <typename T>
 __global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict__ o, const T* __restrict__ proj, int ldp,
@@ -181,14 +366,27 @@ template <typename T>
 static void mlstm_scan_t(const T* proj, int ldp, const float* gate_pre, const int32_t* q_start, const int32_t* pos0,
                          const int32_t* slots, float* S, float* n, float* m, float* a, float* b, float* den, float* o,
                          int B, int H, int D, int Dv, float cap, hipStream_t s) {
-    hy::mlstm_gate_scan_kernel<T><<<dim3(B, H), 64, 0, s>>>(proj, ldp, gate_pre, q_start, pos0, slots, n, m, a, b, den,
-                                                            H, D, cap);
+    // tokens per gate-scan block: as many (<= 64) as keep the staged k and q rows within 40 KB
+    int TG = 64;
+    while (TG > 1 && (size_t)TG * 2 * D * sizeof(T) > 40 * 1024) TG >>= 1;
+    const int gev = 16 / (int)sizeof(T);
+    const int gvec = ldp % gev == 0 && D % gev == 0;  // q and k rows start and end on 16-byte boundaries
+    hy::mlstm_gate_scan_kernel<T><<<dim3(B, H), 256, (size_t)TG * 2 * D * sizeof(T) + 5 * 64 * 4, s>>>(
+        proj, ldp, gate_pre, q_start, pos0, slots, n, m, a, b, den, H, D, cap, TG, gvec);
     const dim3 grid(B, H, (Dv + 63) / 64);
-#define HY_SCAN(DR) hy::mlstm_state_scan_kernel<T, DR><<<grid, 256, 0, s>>>(proj, ldp, a, b, den, q_start, pos0, slots, S, o, H, D, Dv)
+    // rows of q, k, v on 16-byte boundaries: the vector-load kernel with the next stage prefetched (its LDS stays
+    // within the static 64 KB up to D = 256); anything else: the plain one
+    const int ev = 16 / (int)sizeof(T);
+    const bool vec = ldp % ev == 0 && D % ev == 0 && Dv % ev == 0 && D <= 256;
+#define HY_SCAN(DR)                                                                                                    \
+    do {                                                                                                               \
+        if (vec) hy::mlstm_state_scan_vec_kernel<T, DR><<<grid, 256, 0, s>>>(proj, ldp, a, b, den, q_start, pos0, slots, S, o, H, D, Dv); \
+        else hy::mlstm_state_scan_kernel<T, DR><<<grid, 256, 0, s>>>(proj, ldp, a, b, den, q_start, pos0, slots, S, o, H, D, Dv);       \
+    } while (0)
     if (D <= 64) HY_SCAN(16);
     else if (D <= 128) HY_SCAN(32);
     else if (D <= 256) HY_SCAN(64);
-    else HY_SCAN(128);
+    else hy::mlstm_state_scan_kernel<T, 128><<<grid, 256, 0, s>>>(proj, ldp, a, b, den, q_start, pos0, slots, S, o, H, D, Dv);
 #undef HY_SCAN
 }
 

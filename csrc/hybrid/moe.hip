@@ -1,6 +1,7 @@
 // moe.hip — mixture-of-experts feed-forward of the hybrid decoders.
 //
-//   route   per token: float router logits (N = experts + identity outputs), softmax over all N, the `top` largest
+//   route   per token: float router logits (N = experts + identity outputs; the few-row projection of
+//           hybrid_elementwise.hip), then one wave per token: softmax over all N, the `top` largest
 //           of score + correction chosen (the correction steers the choice only), weights = the chosen outputs' plain
 //           scores, not renormalised.  Ties go to the lower index.
 //   ffn     per token: sum over its chosen experts of weight * W_down act(W_up h); an index >= E is an identity
@@ -13,31 +14,20 @@
 namespace chronos {
 namespace hy {
 
-constexpr int kMaxRouterOut = 256;  // N <= 256 (4 per lane)
-
-template <typename T>
-__global__ void __launch_bounds__(256) moe_route_kernel(const T* __restrict__ h, const T* __restrict__ w,
-                                                        const float* __restrict__ corr, int32_t* __restrict__ idx,
-                                                        float* __restrict__ wt, int d, int N, int top) {
-    __shared__ float z[kMaxRouterOut];
-    const int64_t t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const T* hr = h + t * d;
-    for (int r = wv; r < N; r += 4) {
-        const T* wr = w + (int64_t)r * d;
-        float acc = 0.f;
-        for (int k = lane; k < d; k += 64) acc += ld<T>(hr + k) * ld<T>(wr + k);
-        acc = wave_sum(acc);
-        if (lane == 0) z[r] = acc;
-    }
-    __syncthreads();
-    if (wv != 0) return;
+// router outputs N <= 256 (4 per lane)
+// One wave per token: z [T, N] float router logits -> the chosen outputs and their weights.
+__global__ void __launch_bounds__(256) moe_select_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                                                         int32_t* __restrict__ idx, float* __restrict__ wt, int rows,
+                                                         int N, int top) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= rows) return;
     float s[4], c[4];
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int e = lane + 64 * j;
-        s[j] = e < N ? z[e] : -INFINITY;
+        s[j] = e < N ? z[t * N + e] : -INFINITY;
         mx = fmaxf(mx, s[j]);
     }
     mx = wave_max(mx);
@@ -132,11 +122,14 @@ __global__ void __launch_bounds__(256) moe_ffn_token_kernel(const T* __restrict_
 
 }  // namespace hy
 
-void launch_hy_moe_route(const void* h, const void* w, const float* corr, int32_t* idx, float* wt, int T, int d, int N,
-                         int top, bool f32, hipStream_t s) {
+void launch_hy_rowdot(const void*, const void*, const float*, float*, int, int, int, bool, hipStream_t);
+
+// z: float [T, N] scratch for the router logits (the few-row float32-output projection, then the selection)
+void launch_hy_moe_route(const void* h, const void* w, const float* corr, float* z, int32_t* idx, float* wt, int T, int d,
+                         int N, int top, bool f32, hipStream_t s) {
     if (T == 0) return;
-    if (f32) hy::moe_route_kernel<float><<<T, 256, 0, s>>>((const float*)h, (const float*)w, corr, idx, wt, d, N, top);
-    else hy::moe_route_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)h, (const uint16_t*)w, corr, idx, wt, d, N, top);
+    launch_hy_rowdot(h, w, nullptr, z, T, d, N, f32, s);
+    hy::moe_select_kernel<<<(T + 3) / 4, 256, 0, s>>>(z, corr, idx, wt, T, N, top);
 }
 
 void launch_hy_moe_ffn_token(const void* h, const int32_t* idx, const float* wt, const void* w_up, const void* w_down,
