@@ -57,36 +57,72 @@ __global__ void __launch_bounds__(256) layer_norm_kernel(const TY* __restrict__ 
     }
 }
 
-// out[t, n] = sum_k h[t, k] * w[n, k] (+ bias[n]) in float.  One workgroup per TB tokens, whose rows sit in LDS; a
-// wave takes the output rows in turn and reads each weight row ONCE for all TB tokens (the weights are re-read per
-// workgroup from L2, so tokens per workgroup divide that traffic).
-template <typename T, int TB>
+// out[t, n] = sum_k h[t, k] * w[n, k] (+ bias[n]) in float.  A workgroup takes TB tokens (their rows sit in LDS) and
+// 4 output rows, one per wave: a weight row is read ONCE for all TB tokens, 16 bytes per lane when the row length
+// allows (VEC), and the grid's second axis spreads the output rows over workgroups so a handful of decode rows still
+// fills many CUs.
+template <typename T> struct Vec16 { static constexpr int E = 16 / (int)sizeof(T); };
+template <typename T> __device__ __forceinline__ void unpack16(const uint4& v, float* f);
+template <> __device__ __forceinline__ void unpack16<uint16_t>(const uint4& v, float* f) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float(w[i] << 16);
+        f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <> __device__ __forceinline__ void unpack16<float>(const uint4& v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+
+template <typename T, int TB, bool VEC>
 __global__ void __launch_bounds__(256) rowdot_kernel(const T* __restrict__ h, const T* __restrict__ w,
                                                      const float* __restrict__ bias, float* __restrict__ out, int rows,
                                                      int d, int n) {
     extern __shared__ __attribute__((aligned(16))) unsigned char rd_smem[];
     T* hs = reinterpret_cast<T*>(rd_smem);
+    constexpr int E = Vec16<T>::E;
     const int64_t t0 = (int64_t)blockIdx.x * TB;
     const int nt = (int)min((int64_t)TB, rows - t0);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < nt * d; i += 256) hs[i] = h[t0 * d + i];
+    if constexpr (VEC) {
+        const uint4* src = reinterpret_cast<const uint4*>(h + t0 * d);
+        for (int i = threadIdx.x; i < nt * d / E; i += 256) reinterpret_cast<uint4*>(hs)[i] = src[i];
+    } else {
+        for (int i = threadIdx.x; i < nt * d; i += 256) hs[i] = h[t0 * d + i];
+    }
     __syncthreads();
-    for (int r = wv; r < n; r += 4) {
-        const T* wr = w + (int64_t)r * d;
-        float acc[TB];
+    const int r = blockIdx.y * 4 + wv;
+    if (r >= n) return;
+    const T* wr = w + (int64_t)r * d;
+    float acc[TB];
 #pragma unroll
-        for (int u = 0; u < TB; ++u) acc[u] = 0.f;
+    for (int u = 0; u < TB; ++u) acc[u] = 0.f;
+    if constexpr (VEC) {
+        for (int k = lane * E; k < d; k += 64 * E) {
+            float wf[E];
+            unpack16<T>(*reinterpret_cast<const uint4*>(wr + k), wf);
+#pragma unroll
+            for (int u = 0; u < TB; ++u)
+                if (u < nt) {
+                    float hf[E];
+                    unpack16<T>(*reinterpret_cast<const uint4*>(hs + u * d + k), hf);
+#pragma unroll
+                    for (int i = 0; i < E; ++i) acc[u] += hf[i] * wf[i];
+                }
+        }
+    } else {
         for (int k = lane; k < d; k += 64) {
             const float wk = ld<T>(wr + k);
 #pragma unroll
             for (int u = 0; u < TB; ++u)
                 if (u < nt) acc[u] += ld<T>(hs + u * d + k) * wk;
         }
+    }
 #pragma unroll
-        for (int u = 0; u < TB; ++u) {
-            const float v = wave_sum(acc[u]);
-            if (lane == 0 && u < nt) out[(t0 + u) * n + r] = v + (bias != nullptr ? bias[r] : 0.f);
-        }
+    for (int u = 0; u < TB; ++u) {
+        const float v = wave_sum(acc[u]);
+        if (lane == 0 && u < nt) out[(t0 + u) * n + r] = v + (bias != nullptr ? bias[r] : 0.f);
     }
 }
 
@@ -124,17 +160,23 @@ template <typename T>
 static void rowdot_t(const T* h, const T* w, const float* bias, float* out, int rows, int d, int n, hipStream_t s) {
     // tokens per workgroup: as many (up to 8) as keep the staged rows within 48 KB
     const int fit = (48 * 1024) / (d * (int)sizeof(T));
-#define HY_RD(TB)                                                                                              \
-    hy::rowdot_kernel<T, TB><<<(rows + TB - 1) / TB, 256, TB * d * sizeof(T), s>>>(h, w, bias, out, rows, d, n)
+    const bool vec = d % hy::Vec16<T>::E == 0;
+    const int ny = (n + 3) / 4;
+#define HY_RD(TB)                                                                                                  \
+    do {                                                                                                           \
+        const dim3 grid((rows + TB - 1) / TB, ny);                                                                 \
+        if (vec) hy::rowdot_kernel<T, TB, true><<<grid, 256, TB * d * sizeof(T), s>>>(h, w, bias, out, rows, d, n); \
+        else hy::rowdot_kernel<T, TB, false><<<grid, 256, TB * d * sizeof(T), s>>>(h, w, bias, out, rows, d, n);    \
+    } while (0)
     if (fit >= 8 && rows >= 8) HY_RD(8);
     else if (fit >= 4 && rows >= 4) HY_RD(4);
     else if (fit >= 2 && rows >= 2) HY_RD(2);
     else {
-        auto kern = hy::rowdot_kernel<T, 1>;
+        auto kern = hy::rowdot_kernel<T, 1, false>;
         const int bytes = d * (int)sizeof(T);
         if (bytes > 48 * 1024)
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<rows, 256, bytes, s>>>(h, w, bias, out, rows, d, n);
+        kern<<<dim3(rows, ny), 256, bytes, s>>>(h, w, bias, out, rows, d, n);
     }
 #undef HY_RD
 }
