@@ -40,6 +40,7 @@ __global__ void __launch_bounds__(256) mlstm_gate_scan_kernel(
     float* a_s = fg_s + 64;
     float* b_s = a_s + 64;
     float* em_s = b_s + 64;
+    float* dots = em_s + 64;  // [TG][65]: lane l's partial n . q of token t at dots[t * 65 + l]
     // 256 threads stage the block's rows (16-byte loads, 8 in flight per thread); wave 0 runs the recurrences
     const int b = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63;
     const bool w0 = threadIdx.x < 64;
@@ -120,7 +121,8 @@ __global__ void __launch_bounds__(256) mlstm_gate_scan_kernel(
             b_out[(int64_t)(tb + lane) * H + hd] = bb;
         }
         __builtin_amdgcn_wave_barrier();  // wave 0's own LDS writes above, read by its lanes below
-        float den_mine = 0.f;
+        // the n update runs token by token, but no cross-lane reduction sits on that chain: every lane leaves its
+        // partial n . q in LDS, and afterwards lane t adds up token t's 64 partials
         for (int tt = 0; tt < nt; ++tt) {
             const float a = a_s[tt], bb = b_s[tt];
             float dot = 0.f;
@@ -132,10 +134,16 @@ __global__ void __launch_bounds__(256) mlstm_gate_scan_kernel(
                     dot += n[j] * (ld<T>(qst + tt * D + dd) * qs);
                 }
             }
-            dot = wave_sum(dot);
-            if (tt == lane) den_mine = fmaxf(fabsf(dot), em_s[tt]) + 1e-6f;
+            dots[tt * 65 + lane] = dot;
         }
-        if (lane < nt) den_out[(int64_t)(tb + lane) * H + hd] = den_mine;
+        __builtin_amdgcn_wave_barrier();
+        if (lane < nt) {
+            float dsum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int l = 0; l < 64; ++l) dsum[l & 3] += dots[lane * 65 + l];
+            const float dot = (dsum[0] + dsum[1]) + (dsum[2] + dsum[3]);
+            den_out[(int64_t)(tb + lane) * H + hd] = fmaxf(fabsf(dot), em_s[lane]) + 1e-6f;
+        }
     }
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
@@ -312,18 +320,20 @@ __global__ void __launch_bounds__(256) mlstm_state_scan_vec_kernel(
         __syncthreads();
         for (int tt = 0; tt < nt; ++tt) {
             const float a = ab_[tt][0], bv = ab_[tt][1] * vs_[tt][lane];
-            float acc = 0.f;
+            // the wave's DR k and q values: ONE per lane from LDS (two conflict-free reads per token), then handed
+            // to every lane as scalar operands by lane reads — a broadcast LDS read per row costs the LDS pipe a
+            // full 64-lane pass each and was the kernel's limit
+            const int kreg = __float_as_int(ks_[tt][d0 + (lane & (DR - 1))]);
+            const int qreg = __float_as_int(qs_[tt][d0 + (lane & (DR - 1))]);
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};  // independent chains: one wave per SIMD hides no FMA latency
 #pragma unroll
-            for (int j = 0; j < DR; j += 4) {
-                const f32x4 kk = *reinterpret_cast<const f32x4*>(&ks_[tt][d0 + j]);
-                const f32x4 qq = *reinterpret_cast<const f32x4*>(&qs_[tt][d0 + j]);
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    S[j + u] = a * S[j + u] + kk[u] * bv;
-                    acc += S[j + u] * qq[u];
-                }
+            for (int j = 0; j < DR; ++j) {
+                const float kj = __int_as_float(__builtin_amdgcn_readlane(kreg, j));
+                const float qj = __int_as_float(__builtin_amdgcn_readlane(qreg, j));
+                S[j] = a * S[j] + kj * bv;
+                acc[j & 3] += S[j] * qj;
             }
-            part_[wv][tt][lane] = acc;
+            part_[wv][tt][lane] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
         }
         __syncthreads();
         for (int i = threadIdx.x; i < nt * 64; i += 256) {
@@ -371,7 +381,7 @@ static void mlstm_scan_t(const T* proj, int ldp, const float* gate_pre, const in
     while (TG > 1 && (size_t)TG * 2 * D * sizeof(T) > 40 * 1024) TG >>= 1;
     const int gev = 16 / (int)sizeof(T);
     const int gvec = ldp % gev == 0 && D % gev == 0;  // q and k rows start and end on 16-byte boundaries
-    hy::mlstm_gate_scan_kernel<T><<<dim3(B, H), 256, (size_t)TG * 2 * D * sizeof(T) + 5 * 64 * 4, s>>>(
+    hy::mlstm_gate_scan_kernel<T><<<dim3(B, H), 256, (size_t)TG * 2 * D * sizeof(T) + 5 * 64 * 4 + 64 * 65 * 4, s>>>(
         proj, ldp, gate_pre, q_start, pos0, slots, n, m, a, b, den, H, D, cap, TG, gvec);
     const dim3 grid(B, H, (Dv + 63) / 64);
     // rows of q, k, v on 16-byte boundaries: the vector-load kernel with the next stage prefetched (its LDS stays
