@@ -218,8 +218,13 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description="CHRONOS Brain: Ollama-compatible Llama-3 server on MI355X")
     ap.add_argument("--host", default="0.0.0.0")
     ap.add_argument("--port", type=int, default=11434)
-    ap.add_argument("--model", default="llama3-8b", help="preset (random-init) when --checkpoint is not given")
-    ap.add_argument("--checkpoint", default=None, help="HF or Meta Llama-3 checkpoint directory")
+    ap.add_argument("--model", default="llama3-8b",
+                    help="preset of any registered family (random-init) when --checkpoint is not given, e.g. llama3-8b, "
+                         "zokunex-1b; or a checkpoint directory")
+    ap.add_argument("--checkpoint", default=None,
+                    help="checkpoint directory: HF or Meta Llama-3, or a Zokunex config.json + model.safetensors")
+    ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16",
+                    help="activation / weight dtype (fp32: the families that run in it)")
     ap.add_argument("--tokenizer", default=None)
     ap.add_argument("--served-name", default="llama3")
     ap.add_argument("--dp", type=int, default=1, help="engine replicas, one process per GPU")
@@ -251,7 +256,7 @@ def main(argv=None) -> int:
         from ..engine.engine import EngineConfig
 
         cfg = EngineConfig(model=a.model, checkpoint=a.checkpoint, tokenizer=a.tokenizer, device=a.device,
-                           max_slots=a.max_slots, max_model_len=a.max_model_len, kv_dtype=a.kv_dtype,
+                           max_slots=a.max_slots, max_model_len=a.max_model_len, kv_dtype=a.kv_dtype, dtype=a.dtype,
                            request_timeout_s=a.request_timeout, tp_sequence_parallel=a.sequence_parallel)
         if a.tp > 1 or a.cp > 1:
             if a.tp > 1 and a.cp > 1:

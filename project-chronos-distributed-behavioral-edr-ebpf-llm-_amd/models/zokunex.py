@@ -208,7 +208,7 @@ def _preset(width, vocab, pattern, heads, dim, vdim, kv_rank, rot_dim, ff, exper
     layers = []
     for ch in pattern:
         if ch.lower() == "m":
-            mixer, typ = dict(heads=heads, dim=dim, vdim=vdim, gate_cap=15.0), "mlstm"
+            mixer, typ = dict(heads=heads, dim=dim, vdim=vdim, gate_cap=10.0), "mlstm"
         else:
             mixer, typ = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
                               scale=(dim + rot_dim) ** -0.5, rot=dict(base=10000.0, dims=rot_dim)), "latent_attention"

@@ -1,5 +1,5 @@
 """PyTorch references of the hybrid-decoder kernels (csrc/kernels/hybrid*.hip): the CPU execution path and the
-numerics oracle of the GPU tests.  Same contracts as the kernels (layouts, in-place arguments); everything the
+numerics oracle of the GPU tests.  Same interfaces as the kernels (layouts, in-place arguments); everything the
 kernels keep in 32-bit floats is computed in float32 here too, whatever the activation dtype.
 
 Activation dtype ``AT`` is bfloat16 or float32; the residual stream is always float32.

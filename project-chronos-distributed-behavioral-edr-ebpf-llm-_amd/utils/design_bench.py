@@ -2,7 +2,7 @@
 decode steps, and each new kernel beside its closest Llama kernel with the fraction of its roofline it reaches.
 
 ``python bench.py --design-compare [--design-sizes 1k,2k,4k]`` prints one JSON line (the default benchmark and its
-contract are untouched).  Weights are random; every number is measured on the GPU this process runs on.
+output line are untouched).  Weights are random; every number is measured on the GPU this process runs on.
 
 Rooflines: HBM 8 TB/s for kernels bound by the bytes they must move, 2.5 PFLOP/s dense bf16 for the matrix-shaped
 ones (the attention kernels over a long context are priced by their FLOPs in prefill and by their cache bytes in
@@ -33,7 +33,7 @@ def zokunex_config(size: dict) -> dict:
     mh, md, mv = size["m"]
     ah, ad, ar, av, rank = size["a"]
     ne, ni, top, eff = size["moe"]
-    mix_m = dict(type="mlstm", mixer=dict(heads=mh, dim=md, vdim=mv, gate_cap=15.0))
+    mix_m = dict(type="mlstm", mixer=dict(heads=mh, dim=md, vdim=mv, gate_cap=10.0))
     mix_a = dict(type="latent_attention", mixer=dict(heads=ah, dim=ad, rot_dim=ar, vdim=av, kv_rank=rank,
                                                      scale=(ad + ar) ** -0.5, rot=dict(base=10000.0, dims=ar)))
     dense = dict(kind="dense", ff=size["ff"])
@@ -165,11 +165,11 @@ def _kernels(size: dict, dev, T: int, ctx: int, rows: int) -> dict:
     S, n, m = (torch.zeros(NS, mh, md, mv, device=dev), torch.zeros(NS, mh, md, device=dev), torch.zeros(NS, mh, device=dev))
     p0 = torch.zeros(seqs, **i32)
     sl = torch.arange(seqs, **i32)
-    rec("mlstm_scan.prefill", _time(lambda: hops.mlstm_scan(proj, gp, qs, p0, sl, S, n, m, mh, md, mv, 15.0, ctx), iters=3, warm=1),
+    rec("mlstm_scan.prefill", _time(lambda: hops.mlstm_scan(proj, gp, qs, p0, sl, S, n, m, mh, md, mv, 10.0, ctx), iters=3, warm=1),
         nbytes=seqs * ctx * C * 2.0, flops=seqs * ctx * mh * md * mv * 6.0)
     projd, gpd = rnd(rows, C, sc=0.5), rnd(rows, 2 * mh, dt=torch.float32)
     sld = torch.arange(rows, **i32)
-    rec("mlstm_scan.decode", _time(lambda: hops.mlstm_scan(projd, gpd, qsd, posd, sld, S, n, m, mh, md, mv, 15.0, 1)),
+    rec("mlstm_scan.decode", _time(lambda: hops.mlstm_scan(projd, gpd, qsd, posd, sld, S, n, m, mh, md, mv, 10.0, 1)),
         nbytes=rows * mh * md * mv * 4 * 2.0)
     # ---- feed-forwards: the mixture of experts beside a dense SwiGLU of the Llama model at this width
     ne, ni, top, eff = size["moe"]
