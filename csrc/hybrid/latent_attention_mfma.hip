@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         const uint16_t* __restrict__ qa, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_table,
         int max_blocks, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
         const float* __restrict__ gate, uint16_t* __restrict__ out, int H, int DK, int rank, int BS, float scale,
-        int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml) {
+        int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml, int bs_shift) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int b = blockIdx.x;
     const int t0 = q_start[b], t1 = q_start[b + 1];
@@ -39,6 +39,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const int ns = DK / 32, nct = rank / 16;
     const int krs = DK * 2 + 16;            // row-major image: bytes per key row
     const int vts = MKT * 2 + 8;            // transposed image: bytes per value column
+    __shared__ int krow[MKT];  // cache row (page * page size + slot) of each key of the tile
     unsigned char* kimg = smem;
     unsigned char* vimg = smem + MKT * krs;
     // this lane's query row (for the B operand and for the softmax): row r of the sequence, token t0 + r / H
@@ -63,18 +64,41 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     // only known on the device, and a split that gets no tile contributes an empty partial
     for (int k0 = blockIdx.z * MKT; k0 <= pmax; k0 += MKT * nsplit) {
         __syncthreads();
-        // ---- stage: work item = (key pair jp, 8-dim chunk dc); lanes of a wave take consecutive key pairs
-        for (int it = threadIdx.x; it < 32 * chunks; it += 256) {
-            const int jp = it & 31, dc = it >> 5;
-            const int ka = min(k0 + 2 * jp, pmax), kb = min(k0 + 2 * jp + 1, pmax);  // past the end: a real row, masked
-            const u16x8 va = *reinterpret_cast<const u16x8*>(cache + ((int64_t)bt[ka / BS] * BS + ka % BS) * DK + dc * 8);
-            const u16x8 vb = *reinterpret_cast<const u16x8*>(cache + ((int64_t)bt[kb / BS] * BS + kb % BS) * DK + dc * 8);
-            *reinterpret_cast<u16x8*>(kimg + (2 * jp) * krs + dc * 16) = va;
-            *reinterpret_cast<u16x8*>(kimg + (2 * jp + 1) * krs + dc * 16) = vb;
-            if (dc < vchunks) {
+        // ---- cache rows of the tile's 64 keys (page lookup once per key, not once per staged vector: a lookup in
+        // front of every data load made each of them wait for two trips to memory)
+        if (threadIdx.x < MKT) {
+            const int key = min(k0 + (int)threadIdx.x, pmax);  // past the end: a real row, masked below
+            krow[threadIdx.x] = bs_shift >= 0 ? ((bt[key >> bs_shift] << bs_shift) + (key & (BS - 1)))
+                                              : (bt[key / BS] * BS + key % BS);
+        }
+        __syncthreads();
+        // ---- stage: work item = (key pair jp, 8-dim chunk dc); lanes of a wave take consecutive key pairs; three
+        // items' loads (six 16-byte vectors) are issued before any of them is written to LDS
+        for (int it0 = threadIdx.x; it0 < 32 * chunks; it0 += 256 * 3) {
+            u16x8 va[3], vb[3];
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    *reinterpret_cast<uint32_t*>(vimg + (dc * 8 + e) * vts + jp * 4) = (uint32_t)va[e] | ((uint32_t)vb[e] << 16);
+            for (int u = 0; u < 3; ++u) {
+                const int it = it0 + 256 * u;
+                if (it < 32 * chunks) {
+                    const int jp = it & 31, dc = it >> 5;
+                    va[u] = *reinterpret_cast<const u16x8*>(cache + (int64_t)krow[2 * jp] * DK + dc * 8);
+                    vb[u] = *reinterpret_cast<const u16x8*>(cache + (int64_t)krow[2 * jp + 1] * DK + dc * 8);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 3; ++u) {
+                const int it = it0 + 256 * u;
+                if (it < 32 * chunks) {
+                    const int jp = it & 31, dc = it >> 5;
+                    *reinterpret_cast<u16x8*>(kimg + (2 * jp) * krs + dc * 16) = va[u];
+                    *reinterpret_cast<u16x8*>(kimg + (2 * jp + 1) * krs + dc * 16) = vb[u];
+                    if (dc < vchunks) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            *reinterpret_cast<uint32_t*>(vimg + (dc * 8 + e) * vts + jp * 4) =
+                                (uint32_t)va[u][e] | ((uint32_t)vb[u][e] << 16);
+                    }
+                }
             }
         }
         __syncthreads();
@@ -104,13 +128,13 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(mrow, mx);
-        const float corr = (mn == -INFINITY) ? 1.f : expf(mrow - mn);
+        const float corr = (mn == -INFINITY) ? 1.f : __expf(mrow - mn);
         float sum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = (mn == -INFINITY) ? 0.f : expf(S[kt][i] - mn);
+                const float p = (mn == -INFINITY) ? 0.f : __expf(S[kt][i] - mn);
                 S[kt][i] = p;
                 sum += p;
             }
@@ -203,8 +227,9 @@ static void la_mfma_launch(const uint16_t* qa, const uint16_t* cache, const int3
         set_bytes = bytes;
     }
     const dim3 grid(B, (max_q * H + 63) / 64, nsplit);
+    const int bs_shift = (BS & (BS - 1)) == 0 ? __builtin_ctz(BS) : -1;
     kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale, nsplit, part_o,
-                                  part_ml);
+                                  part_ml, bs_shift);
 }
 
 bool hy_latent_mfma_ok(int DK, int rank) { return !(DK % 32 || rank % 16 || DK > 576 || rank > 512 || rank > DK); }
