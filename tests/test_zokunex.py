@@ -322,3 +322,48 @@ def test_registry_reads_the_checkpoint_layout(tmp_path):
         zokunex.config_from_dict(bad)
     with pytest.raises(NotImplementedError):
         registry.build_model("tiny", "cpu", dtype="fp32")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_compaction_and_preemption_carry_the_state(device):
+    """Requests that finish at different times leave holes in the low slots, so running sequences are moved down
+    (their recurrent state has to move with them); a page pool too small for all of them forces recompute
+    preemption (the sequence re-prefills prompt + generated tokens from position 0, which rebuilds its state).
+    Greedy tokens must equal the oracle's throughout."""
+    cfg = _config([(_mlstm(heads=2, dim=8, vdim=8), _dense(32)), (_latent(), _moe(3, 1, 2, 16))], width=32, vocab=61, logit_scale=4.0)
+    prompts = [_tokens(n, 59, 50 + n) for n in (4, 6, 9, 30)]
+    budgets = [3, 5, 24, 26]
+    # compaction: four slots, the two short requests finish first and the two long ones are moved into their slots
+    eng, tensors = _engine(cfg, device, slots=4, max_len=96, use_graphs=False, decode_burst=2, prefill_ramp=0)
+    reqs = [eng.submit(p, num_predict=n) for p, n in zip(prompts, budgets)]
+    eng.run_until_idle(max_steps=2000)
+    assert eng.stats["compactions"] >= 1
+    for r, p, n in zip(reqs, prompts, budgets):
+        want = _greedy(cfg, tensors, p, n)
+        assert len(r.out_ids) >= n - 1 and r.out_ids == want[:len(r.out_ids)], (r.out_ids, want)
+    # preemption: lazy page growth over a pool of 5 usable pages; the two long requests end up needing 6
+    eng, _ = _engine(cfg, device, slots=4, max_len=96, blocks=6, tensors=tensors, use_graphs=False, decode_burst=2,
+                     prefill_ramp=0, kv_alloc="lazy", kv_lookahead=2, kv_watermark=0.0)
+    reqs = [eng.submit(p, num_predict=n) for p, n in zip(prompts, budgets)]
+    eng.run_until_idle(max_steps=4000)
+    assert eng.stats["preemptions"] >= 1
+    for r, p, n in zip(reqs, prompts, budgets):
+        assert r.done_reason in ("length", "stop"), (r.done_reason, r.error)
+        want = _greedy(cfg, tensors, p, n)
+        assert len(r.out_ids) >= n - 1 and r.out_ids == want[:len(r.out_ids)], (r.out_ids, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("width", [512, 1024])
+def test_wide_model_decode_rows_on_the_routed_projections(width):
+    """Widths at which single decode rows take the framework's GEMV (K % 512 == 0) and the experts the grouped MFMA
+    GEMMs (widths on the 128 grid): bfloat16 prefill against token-by-token decoding against the oracle."""
+    cfg = _config([(_mlstm(heads=2, dim=64, vdim=128), _moe(4, 1, 2, 128)),
+                   (_latent(heads=4, dim=32, rot_dim=32, dims=32, vdim=64, rank=96, scale=0.125), _dense(1024))],
+                  width=width, vocab=320)
+    eng, tensors = _engine(cfg, "cuda", "bf16", max_len=128)
+    toks = _tokens(40, 320, 3)
+    want = plain.forward(cfg, tensors, toks)
+    for sched in ([[("r0", 40)]], [[("r0", 9)]] + [[("r0", 1)] for _ in range(31)]):
+        got = _replay(eng, sched, {"r0": toks})["r0"].cpu()
+        assert not _bad(got, want, "bf16"), _errs(got, want)
