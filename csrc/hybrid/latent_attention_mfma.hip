@@ -15,16 +15,22 @@
 //     fixed permutation of the 32 keys, the same one the transposed value image is read with), so the weights never
 //     leave registers.  Accumulators: rank / 16 tiles x 4 registers.
 // Sizes: DK % 32 == 0, rank % 16 == 0, DK <= 576, rank <= 512.  Everything else takes latent_attention.hip.
+#include <cstdlib>
+
 #include "hybrid_common.h"
 
 namespace chronos {
 namespace hy {
 
-constexpr int MKT = 64;  // keys per tile
+constexpr int MKT = 64;  // keys per tile at most
 
-// NS: k-steps of the scores (DK / 32) at most; NCT: 16-column tiles of the output (rank / 16) at most.
-template <int NS, int NCT>
-__global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
+// NS: k-steps of the scores (DK / 32) at most; NCT: 16-column tiles of the output (rank / 16) at most; KT: keys per
+// tile, 64 or 32 (32 halves the LDS images, so two workgroups share a CU at the widest rows and one stages while the
+// other multiplies).
+// NW: waves per workgroup, 4 or 8 (16 query rows each): with 8 a staged key tile serves 128 rows and every SIMD holds two
+// waves, so one wave's softmax and staging run beside the other's MFMAs.
+template <int NS, int NCT, int KT, int NW>
+__global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
         const uint16_t* __restrict__ qa, const uint16_t* __restrict__ cache, const int32_t* __restrict__ block_table,
         int max_blocks, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
         const float* __restrict__ gate, uint16_t* __restrict__ out, int H, int DK, int rank, int BS, float scale,
@@ -33,22 +39,24 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const int b = blockIdx.x;
     const int t0 = q_start[b], t1 = q_start[b + 1];
     const int rows_total = (t1 - t0) * H;
-    const int rb0 = blockIdx.y * 64;
+    constexpr int NT = 64 * NW, RPB = 16 * NW;  // threads and query rows per workgroup
+    const int rb0 = blockIdx.y * RPB;
     if (rb0 >= rows_total) return;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, g = lane >> 4, qi = lane & 15;
     const int ns = DK / 32, nct = rank / 16;
     const int krs = DK * 2 + 16;            // row-major image: bytes per key row
-    const int vts = MKT * 2 + 8;            // transposed image: bytes per value column
+    constexpr int vts = KT * 2 + 8;         // transposed image: bytes per value column
+    constexpr int PP = KT / 2;              // key pairs per tile
     __shared__ int krow[MKT];  // cache row (page * page size + slot) of each key of the tile
     unsigned char* kimg = smem;
-    unsigned char* vimg = smem + MKT * krs;
+    unsigned char* vimg = smem + KT * krs;
     // this lane's query row (for the B operand and for the softmax): row r of the sequence, token t0 + r / H
     const int r = rb0 + wv * 16 + qi;
     const bool rok = r < rows_total;
     const int rc = rok ? r : rows_total - 1;
     const int64_t grow = (int64_t)t0 * H + rc;              // row of qa / out / gate
     const int prow = rok ? pos[t0 + rc / H] : -1;
-    const int last_row = min(rows_total, rb0 + 64) - 1;
+    const int last_row = min(rows_total, rb0 + RPB) - 1;
     const int pmax = pos[t0 + last_row / H];                // positions grow along the sequence
     bf16x8 qf[NS];
 #pragma unroll
@@ -62,11 +70,11 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const int chunks = DK / 8, vchunks = rank / 8;
     // key tiles are dealt round-robin to the nsplit workgroups of this row block (blockIdx.z): the context length is
     // only known on the device, and a split that gets no tile contributes an empty partial
-    for (int k0 = blockIdx.z * MKT; k0 <= pmax; k0 += MKT * nsplit) {
+    for (int k0 = blockIdx.z * KT; k0 <= pmax; k0 += KT * nsplit) {
         __syncthreads();
         // ---- cache rows of the tile's 64 keys (page lookup once per key, not once per staged vector: a lookup in
         // front of every data load made each of them wait for two trips to memory)
-        if (threadIdx.x < MKT) {
+        if (threadIdx.x < KT) {
             const int key = min(k0 + (int)threadIdx.x, pmax);  // past the end: a real row, masked below
             krow[threadIdx.x] = bs_shift >= 0 ? ((bt[key >> bs_shift] << bs_shift) + (key & (BS - 1)))
                                               : (bt[key / BS] * BS + key % BS);
@@ -74,22 +82,22 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         __syncthreads();
         // ---- stage: work item = (key pair jp, 8-dim chunk dc); lanes of a wave take consecutive key pairs; three
         // items' loads (six 16-byte vectors) are issued before any of them is written to LDS
-        for (int it0 = threadIdx.x; it0 < 32 * chunks; it0 += 256 * 3) {
+        for (int it0 = threadIdx.x; it0 < PP * chunks; it0 += NT * 3) {
             u16x8 va[3], vb[3];
 #pragma unroll
             for (int u = 0; u < 3; ++u) {
-                const int it = it0 + 256 * u;
-                if (it < 32 * chunks) {
-                    const int jp = it & 31, dc = it >> 5;
+                const int it = it0 + NT * u;
+                if (it < PP * chunks) {
+                    const int jp = it & (PP - 1), dc = it / PP;
                     va[u] = *reinterpret_cast<const u16x8*>(cache + (int64_t)krow[2 * jp] * DK + dc * 8);
                     vb[u] = *reinterpret_cast<const u16x8*>(cache + (int64_t)krow[2 * jp + 1] * DK + dc * 8);
                 }
             }
 #pragma unroll
             for (int u = 0; u < 3; ++u) {
-                const int it = it0 + 256 * u;
-                if (it < 32 * chunks) {
-                    const int jp = it & 31, dc = it >> 5;
+                const int it = it0 + NT * u;
+                if (it < PP * chunks) {
+                    const int jp = it & (PP - 1), dc = it / PP;
                     *reinterpret_cast<u16x8*>(kimg + (2 * jp) * krs + dc * 16) = va[u];
                     *reinterpret_cast<u16x8*>(kimg + (2 * jp + 1) * krs + dc * 16) = vb[u];
                     if (dc < vchunks) {
@@ -102,10 +110,11 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
             }
         }
         __syncthreads();
-        // ---- scores: 4 key tiles of 16; lane gets keys 16 kt + 4 g + i of query row qi
-        f32x4 S[4];
+        // ---- scores: KT / 16 key tiles of 16; lane gets keys 16 kt + 4 g + i of query row qi
+        constexpr int NKT = KT / 16;
+        f32x4 S[NKT];
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
+        for (int kt = 0; kt < NKT; ++kt) {
             S[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
             const unsigned char* arow = kimg + (16 * kt + qi) * krs + g * 16;
 #pragma unroll
@@ -117,7 +126,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         // ---- softmax over the tile for query row qi (this lane and the 3 other lane groups hold its keys)
         float mx = -INFINITY;
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = k0 + 16 * kt + 4 * g + i;
@@ -131,7 +140,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         const float corr = (mn == -INFINITY) ? 1.f : __expf(mrow - mn);
         float sum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float p = (mn == -INFINITY) ? 0.f : __expf(S[kt][i] - mn);
@@ -143,9 +152,10 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         lrow = lrow * corr + sum;
         mrow = mn;
         // ---- weighted sum of the value columns: k index of step u = [tile 2u keys 4g..4g+3 | tile 2u+1 keys 4g..4g+3]
-        bf16x8 pf[2];
+        constexpr int NU = KT / 32;
+        bf16x8 pf[NU];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < NU; ++u)
             pf[u] = bf16x8{(__bf16)S[2 * u][0], (__bf16)S[2 * u][1], (__bf16)S[2 * u][2], (__bf16)S[2 * u][3],
                            (__bf16)S[2 * u + 1][0], (__bf16)S[2 * u + 1][1], (__bf16)S[2 * u + 1][2], (__bf16)S[2 * u + 1][3]};
 #pragma unroll
@@ -154,7 +164,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
                 O[c] *= corr;
                 const unsigned char* vrow = vimg + (16 * c + qi) * vts + g * 8;
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < NU; ++u) {
                     const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow + u * 64);
                     const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + u * 64 + 32);
                     const bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -214,21 +224,21 @@ __global__ void __launch_bounds__(256) latent_combine_kernel(const float* __rest
 
 }  // namespace hy
 
-template <int NS, int NCT>
+template <int NS, int NCT, int KT, int NW>
 static void la_mfma_launch(const uint16_t* qa, const uint16_t* cache, const int32_t* bt, int max_blocks,
                            const int32_t* q_start, const int32_t* pos, const float* gate, uint16_t* out, int B, int H,
                            int DK, int rank, int BS, int max_q, float scale, int nsplit, float* part_o, float* part_ml,
                            hipStream_t s) {
-    auto kern = hy::latent_attention_mfma_kernel<NS, NCT>;
-    const int bytes = hy::MKT * (DK * 2 + 16) + rank * (hy::MKT * 2 + 8);
+    auto kern = hy::latent_attention_mfma_kernel<NS, NCT, KT, NW>;
+    const int bytes = KT * (DK * 2 + 16) + rank * (KT * 2 + 8);
     static int set_bytes = 0;
     if (bytes > set_bytes) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         set_bytes = bytes;
     }
-    const dim3 grid(B, (max_q * H + 63) / 64, nsplit);
+    const dim3 grid(B, (max_q * H + 16 * NW - 1) / (16 * NW), nsplit);
     const int bs_shift = (BS & (BS - 1)) == 0 ? __builtin_ctz(BS) : -1;
-    kern<<<grid, 256, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale, nsplit, part_o,
+    kern<<<grid, 64 * NW, bytes, s>>>(qa, cache, bt, max_blocks, q_start, pos, gate, out, H, DK, rank, BS, scale, nsplit, part_o,
                                   part_ml, bs_shift);
 }
 
@@ -252,10 +262,23 @@ bool launch_hy_latent_attention_mfma(const uint16_t* qa, const uint16_t* cache, 
                                      float* part_ml, int64_t total_rows, hipStream_t s) {
     if (!hy_latent_mfma_ok(DK, rank)) return false;
     if (B == 0 || max_q == 0) return true;
-#define HY_LAM(NS, NCT) la_mfma_launch<NS, NCT>(qa, cache, bt, max_blocks, q_start, pos, gate, out, B, H, DK, rank, BS, max_q, scale, nsplit, part_o, part_ml, s)
-    if (DK <= 128 && rank <= 64) HY_LAM(4, 4);
-    else if (DK <= 320 && rank <= 256) HY_LAM(10, 16);
-    else HY_LAM(18, 32);
+#define HY_LAM(NS, NCT, KT, NW) la_mfma_launch<NS, NCT, KT, NW>(qa, cache, bt, max_blocks, q_start, pos, gate, out, B, H, DK, rank, BS, max_q, scale, nsplit, part_o, part_ml, s)
+    // 64-key tiles (32-key tiles measured slower at every size: the per-tile softmax and barriers weigh more than the
+    // second workgroup per CU gains; CHRONOS_LATENT_KT=32 keeps them for A/B).  8 waves per workgroup when a sequence
+    // brings more than 64 rows (CHRONOS_LATENT_NW=4 / 8 forces one).
+    static const int force_kt = [] { const char* v = getenv("CHRONOS_LATENT_KT"); return v ? atoi(v) : 0; }();
+    static const int force_nw = [] { const char* v = getenv("CHRONOS_LATENT_NW"); return v ? atoi(v) : 0; }();
+    const bool kt32 = force_kt == 32;
+    const bool nw8 = force_nw == 8 || (force_nw != 4 && max_q * H > 64);
+#define HY_LAM_T(NS, NCT)                                                            \
+    do {                                                                             \
+        if (kt32) { if (nw8) HY_LAM(NS, NCT, 32, 8); else HY_LAM(NS, NCT, 32, 4); }   \
+        else { if (nw8) HY_LAM(NS, NCT, 64, 8); else HY_LAM(NS, NCT, 64, 4); }       \
+    } while (0)
+    if (DK <= 128 && rank <= 64) HY_LAM_T(4, 4);
+    else if (DK <= 320 && rank <= 256) HY_LAM_T(10, 16);
+    else HY_LAM_T(18, 32);
+#undef HY_LAM_T
 #undef HY_LAM
     if (nsplit > 1)
         hy::latent_combine_kernel<<<(unsigned)((total_rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, gate, out, total_rows, rank, nsplit);
