@@ -359,7 +359,7 @@ def test_wide_model_decode_rows_on_the_routed_projections(width):
     """Widths at which single decode rows take the framework's GEMV (K % 512 == 0) and the experts the grouped MFMA
     GEMMs (widths on the 128 grid): bfloat16 prefill against token-by-token decoding against the oracle."""
     cfg = _config([(_mlstm(heads=2, dim=64, vdim=128), _moe(4, 1, 2, 128)),
-                   (_latent(heads=4, dim=32, rot_dim=32, dims=32, vdim=64, rank=96, scale=0.125), _dense(1024))],
+                   (_latent(heads=4, dim=48, rot_dim=32, dims=32, vdim=64, rank=96, scale=0.1), _dense(1024))],
                   width=width, vocab=320)
     eng, tensors = _engine(cfg, "cuda", "bf16", max_len=128)
     toks = _tokens(40, 320, 3)
