@@ -1,6 +1,8 @@
 """Hybrid decoders: a list of layers, each with a token mixer of some kind (recurrent matrix memory, latent
-attention) and an optional feed-forward (dense, mixture of experts), on a float32 residual stream with the norm on the
-sublayer's OUTPUT (x <- x + norm(sublayer(x))).
+attention, windowed attention with sinks, gated delta rule, gated linear attention) and an optional feed-forward
+(dense, gated, mixture of experts), on a float32 residual stream.  The stream's rule is a parameter of the
+configuration: the norm on the sublayer's OUTPUT (``out_norm``: x <- x + layer_norm(sublayer(x))) or AFTER the sum
+(``post_norm``: x <- rms_norm(alpha x + sublayer(x))).
 
 This module is the design-independent part: the mixer and feed-forward kinds with their sizes and constants as
 parameters, the cache that holds pages for the attention layers and state slots for the recurrent ones, and the
@@ -70,6 +72,87 @@ class MoEFFSpec:
 
 
 @dataclass
+class WindowAttentionSpec:
+    """Grouped-query softmax attention through a sliding window that also keeps each sequence's first tokens, with
+    per-head RMS norm of queries and keys, rotation of the leading ``rope_dims`` columns (long wavelengths slowed
+    down by ``rope_scaling`` = (factor, low, high, original length)), a learned softmax sink per head, an optional
+    mix of every token's values with those of the first such layer, and a sigmoid output gate per head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0          # 0: every earlier token is visible
+    keep_first: int = 0      # tokens at positions below this stay visible past the window
+    rope_base: float = 10000.0
+    rope_dims: int = 0       # 0: no rotation
+    rope_scaling: Optional[tuple] = None
+    v_mix: bool = False
+    v_mix_first: bool = False  # this layer is the source of the mixed-in values (and does not mix itself)
+    kind: str = "window_attention"
+
+    def params(self, d: int) -> int:
+        return d * (self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + self.heads) + 2 * self.dim + \
+            self.heads + 1 + self.heads * self.vdim * d
+
+
+@dataclass
+class DeltaRuleSpec:
+    """Gated delta rule: per value head a dim x vdim state that decays, is corrected towards the current value along
+    the current (unit) key, and is read by the (unit) query; q, k, v pass a short causal convolution and SiLU."""
+    heads: int
+    kv_heads: int   # query / key heads (value head h reads head h // (heads / kv_heads))
+    dim: int
+    vdim: int
+    conv: int
+    kind: str = "delta_rule"
+
+    def params(self, d: int) -> int:
+        c = 2 * self.kv_heads * self.dim + self.heads * self.vdim
+        return c * (d + self.conv) + self.heads * (2 * d + 2) + self.vdim + 2 * self.heads * self.vdim * d
+
+
+@dataclass
+class GLASpec:
+    """Gated linear attention: per head a dim x vdim state whose rows decay by sigmoid(z)^(1/tau), z a low-rank
+    projection of the input with a bias."""
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    rank: int
+    kind: str = "gla"
+
+    def params(self, d: int) -> int:
+        hd, hv = self.heads * self.dim, self.heads * self.vdim
+        return d * (2 * hd + 2 * hv) + self.rank * (d + hd) + hd + self.vdim + hv * d
+
+
+@dataclass
+class GluFFSpec:
+    """Gated feed-forward: y = g sigmoid(slope g) (u + shift) with g = min(W_gate h, limit) and
+    u = clamp(W_up h, -limit, limit)."""
+    ff: int
+    limit: float
+    slope: float = 1.702
+    shift: float = 1.0
+    kind: str = "glu"
+
+
+@dataclass
+class MoEGluSpec:
+    """Mixture of gated experts; the router adds a bias to its logits, takes the ``top`` largest and weighs them by
+    the softmax over the chosen logits only."""
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    slope: float = 1.702
+    shift: float = 1.0
+    kind: str = "moe_glu"
+
+
+@dataclass
 class LayerSpec:
     mixer: object
     ff: Optional[object]
@@ -85,24 +168,32 @@ class HybridConfig:
     logit_scale: float = 1.0
     max_position: int = 8192
     architecture: str = "hybrid"
+    residual: str = "out_norm"     # "out_norm": x <- x + layer_norm(y);  "post_norm": x <- rms_norm(alpha x + y)
+    residual_alpha: float = 1.0
+    tied_head: bool = False        # the logits come from the embedding table
 
     @property
     def num_layers(self) -> int:
         return len(self.layers)
 
     def param_count(self) -> int:
-        d, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size + self.hidden_size
+        d = self.hidden_size
+        n = (1 if self.tied_head else 2) * self.vocab_size * d + d
         for l in self.layers:
             m = l.mixer
-            if m.kind == "mlstm":
+            if hasattr(m, "params"):
+                n += m.params(d)
+            elif m.kind == "mlstm":
                 n += d * (2 * m.heads * m.dim + 2 * m.heads * m.vdim) + 2 * m.heads * (d + 1) + m.heads * m.vdim * (d + 1)
             else:
                 n += d * (m.heads * (m.dim + m.rot_dim) + m.kv_rank + m.rot_dim + m.heads) + m.kv_rank
                 n += m.kv_rank * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * d
             n += d
             if l.ff is not None:
-                n += d + (2 * d * l.ff.ff if l.ff.kind == "dense" else
-                          l.ff.experts * 2 * d * l.ff.ff + (l.ff.experts + l.ff.identity) * (d + 1))
+                f = l.ff
+                n += d + {"dense": lambda: 2 * d * f.ff, "glu": lambda: 3 * d * f.ff,
+                          "moe": lambda: f.experts * 2 * d * f.ff + (f.experts + f.identity) * (d + 1),
+                          "moe_glu": lambda: f.experts * (3 * d * f.ff + d + 1)}[f.kind]()
         return n
 
 
@@ -112,9 +203,12 @@ class HybridConfig:
 
 
 class HybridCache:
-    """Per attention layer a paged latent cache [NB, BS, kv_rank + rot_dim] in the activation dtype (block 0 is the
-    engine's scratch block); per recurrent layer float32 state rows S [NS, H, D, Dv], n [NS, H, D], m [NS, H], one row
-    per engine slot plus a scratch row (``scratch_slot``) for the decode rows of slots that hold no running sequence.
+    """Per latent-attention layer a paged latent cache [NB, BS, kv_rank + rot_dim], per windowed-attention layer
+    paged keys [NB, BS, G, D] and values [NB, BS, G, Dv], all in the activation dtype (block 0 is the engine's scratch
+    block); per recurrent layer float32 state rows S [NS, H, D, Dv] (the matrix-memory layers also n [NS, H, D] and
+    m [NS, H]; the delta-rule layers also the last conv - 1 inputs of their convolution, ``hist`` [NS, conv - 1, C] in
+    the activation dtype), one row per engine slot plus a scratch row (``scratch_slot``) for the decode rows of slots
+    that hold no running sequence.
 
     A sequence's state needs no reset: a step whose first token sits at position 0 starts from zero."""
 
@@ -126,6 +220,9 @@ class HybridCache:
         self.S: dict[int, torch.Tensor] = {}
         self.n: dict[int, torch.Tensor] = {}
         self.m: dict[int, torch.Tensor] = {}
+        self.kc: dict[int, torch.Tensor] = {}
+        self.vc: dict[int, torch.Tensor] = {}
+        self.hist: dict[int, torch.Tensor] = {}
         for li, l in enumerate(cfg.layers):
             mx = l.mixer
             if mx.kind == "latent_attention":
@@ -136,16 +233,31 @@ class HybridCache:
                 self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, **f32)
                 self.n[li] = torch.zeros(slots + 1, mx.heads, mx.dim, **f32)
                 self.m[li] = torch.zeros(slots + 1, mx.heads, **f32)
+            elif mx.kind == "window_attention":
+                pg = dict(device=device, dtype=act_dtype)
+                self.kc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.dim, **pg)
+                self.vc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.vdim, **pg)
+            elif mx.kind in ("delta_rule", "gla"):
+                self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, device=device, dtype=torch.float32)
+                if mx.kind == "delta_rule":
+                    ch = 2 * mx.kv_heads * mx.dim + mx.heads * mx.vdim
+                    self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), ch, device=device, dtype=act_dtype)
 
     @staticmethod
     def bytes_per_block(cfg: HybridConfig, block_size: int, act_dtype) -> int:
         eb = 4 if act_dtype == torch.float32 else 2
-        return max(1, sum(block_size * (l.mixer.kv_rank + l.mixer.rot_dim) * eb for l in cfg.layers
-                          if l.mixer.kind == "latent_attention"))
+        per_token = 0
+        for l in cfg.layers:
+            m = l.mixer
+            if m.kind == "latent_attention":
+                per_token += m.kv_rank + m.rot_dim
+            elif m.kind == "window_attention":
+                per_token += m.kv_heads * (m.dim + m.vdim)
+        return max(1, block_size * per_token * eb)
 
     def move_slots(self, src: torch.Tensor, dst: torch.Tensor) -> None:
         """Slot compaction: the recurrent state rows follow their sequences."""
-        for t in (*self.S.values(), *self.n.values(), *self.m.values()):
+        for t in (*self.S.values(), *self.n.values(), *self.m.values(), *self.hist.values()):
             t.index_copy_(0, dst, t.index_select(0, src))
 
 
@@ -213,10 +325,67 @@ def pack_moe(spec: MoEFFSpec, t: dict, device, act_dtype) -> dict:
                 w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
 
 
-def rope_cos_sin(base: float, dims: int, max_pos: int, device) -> torch.Tensor:
+def pack_window_attention(spec: WindowAttentionSpec, t: dict, device, act_dtype) -> dict:
+    """t: q, k, v, q.norm, k.norm, sink, g, o and, in value-mixing layers, vmix.  q | k | v become one projection;
+    the per-head gate rows are a few-row float32-output projection."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    out = dict(w_qkv=a(torch.cat([t["q"], t["k"], t["v"]], 0)), q_norm=f(t["q.norm"]), k_norm=f(t["k.norm"]),
+               sink=f(t["sink"]), w_g=a(t["g"]), w_o=a(t["o"]))
+    if spec.v_mix and not spec.v_mix_first:
+        out["vmix"] = f(t["vmix"]).reshape(1)
+    return out
+
+
+def pack_delta_rule(spec: DeltaRuleSpec, t: dict, device, act_dtype) -> dict:
+    """t: q, k, v (+ .conv each), b, a, dt_bias, A_log, g, norm, o.  q | k | v | g are one projection, the
+    convolution taps of q | k | v one [C, conv] float32 table, decay and write-strength rows one few-row
+    float32-output projection (bias: dt_bias for the decay rows, zero for the others)."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    return dict(w_proj=a(torch.cat([t["q"], t["k"], t["v"], t["g"]], 0)),
+                taps=f(torch.cat([t["q.conv"], t["k.conv"], t["v.conv"]], 0)),
+                w_ab=a(torch.cat([t["a"], t["b"]], 0)),
+                b_ab=f(torch.cat([t["dt_bias"].float(), torch.zeros(spec.heads)], 0)), a_log=f(t["A_log"]),
+                norm=f(t["norm"].float().repeat(spec.heads)), w_o=a(t["o"]))
+
+
+def pack_gla(spec: GLASpec, t: dict, device, act_dtype) -> dict:
+    """t: q, k, v, g, a1, a2, a2.b, norm, o.  q | k | v | g are one projection; the decay's low-rank projection keeps
+    float32 outputs (a1 through the few-row projection, a2 as a float32 matrix)."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    return dict(w_proj=a(torch.cat([t["q"], t["k"], t["v"], t["g"]], 0)), w_a1=a(t["a1"]), w_a2t=f(t["a2"].float().t()),
+                b_a2=f(t["a2.b"]), norm=f(t["norm"].float().repeat(spec.heads)), w_o=a(t["o"]))
+
+
+def pack_glu(spec: GluFFSpec, t: dict, device, act_dtype) -> dict:
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    return dict(w_gu=a(torch.cat([t["gate"], t["up"]], 0)), w_down=a(t["down"]))
+
+
+def pack_moe_glu(spec: MoEGluSpec, t: dict, device, act_dtype) -> dict:
+    """t: router, router.b, e<k>.gate, e<k>.up, e<k>.down.  Per expert gate rows then up rows, stacked [E, 2F, d]."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    return dict(w_router=a(t["router"]), b_router=t["router.b"].to(device=device, dtype=torch.float32).contiguous(),
+                w_gu=a(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(spec.experts)])),
+                w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
+
+
+def rope_cos_sin(base: float, dims: int, max_pos: int, device, scaling: Optional[tuple] = None) -> torch.Tensor:
     """[max_pos, dims] float32: cos(p f_i) for i < dims/2, then sin(p f_i), f_i = base^(-2i/dims); angles in float64
-    before the rounding to float32."""
+    before the rounding to float32.  ``scaling`` = (factor, low, high, original): frequencies whose wavelength is
+    shorter than original/high stay, those longer than original/low are divided by factor, and between the two the
+    frequency is interpolated linearly in original/wavelength."""
     inv = base ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
+    if scaling is not None:
+        import math
+
+        factor, low, high, orig = (float(v) for v in scaling)
+        wl = 2 * math.pi / inv
+        s = ((orig / wl - low) / (high - low)).clamp(0.0, 1.0) if high != low else torch.ones_like(inv)
+        mid = (1 - s) * inv / factor + s * inv
+        inv = torch.where(wl < orig / high, inv, torch.where(wl > orig / low, inv / factor, mid))
     fr = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
     return torch.cat([fr.cos(), fr.sin()], 1).float().to(device)
 
@@ -240,6 +409,7 @@ class StepMeta:
     slots: torch.Tensor
     last_idx: torch.Tensor
     max_q: int
+    shared: dict = field(default_factory=dict)  # what one layer of a step leaves for later layers of the same step
 
 
 def mix_mlstm(model, li: int, spec: MLSTMSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
@@ -271,6 +441,54 @@ def mix_latent_attention(model, li: int, spec: LatentAttentionSpec, w: dict, h, 
     return hops.matmul(ov, w["w_o"])
 
 
+def mix_window_attention(model, li: int, spec: WindowAttentionSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    H, G, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    qkv = hops.matmul(h, w["w_qkv"])
+    gate = hops.rowdot(h, w["w_g"])
+    mixes = spec.v_mix and not spec.v_mix_first
+    v = hops.window_prep(qkv, H, G, D, Dv, meta.shared["v_first"] if mixes else None, w.get("vmix"), meta.pos,
+                         meta.tok_seq, meta.block_table, w["q_norm"], w["k_norm"], model.cfg.norm_eps,
+                         model.rope.get(li), spec.rope_dims, cache.kc[li], cache.vc[li], spec.v_mix_first)
+    if spec.v_mix_first:
+        meta.shared["v_first"] = v
+    o = hops.window_attention(qkv, cache.kc[li], cache.vc[li], meta.block_table, meta.q_start, meta.pos, w["sink"],
+                              gate, spec.scale, spec.window, spec.keep_first, H, model.act_dtype, meta.max_q)
+    return hops.matmul(o, w["w_o"])
+
+
+def mix_delta_rule(model, li: int, spec: DeltaRuleSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    H, HK, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    C = 2 * HK * D + H * Dv
+    proj = hops.matmul(h, w["w_proj"])          # q | k | v | g
+    ab = hops.rowdot(h, w["w_ab"], w["b_ab"])   # decay and write-strength pre-activations, float32
+    y = hops.short_conv(proj, w["taps"], meta.q_start, meta.pos0, meta.slots, cache.hist[li], True)
+    qscale, kscale, decay, beta = hops.delta_prep(y, ab, w["a_log"], HK, H, D, D ** -0.5)
+    o = hops.linear_scan(y, 0, HK * D, 2 * HK * D, qscale, kscale, 1.0, decay, beta, meta.q_start, meta.pos0,
+                         meta.slots, cache.S[li], HK, H, D, Dv)
+    return hops.matmul(hops.head_norm_gate(o, proj, C, w["norm"], model.cfg.norm_eps, True, model.act_dtype), w["w_o"])
+
+
+def mix_gla(model, li: int, spec: GLASpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    H, D, Dv = spec.heads, spec.dim, spec.vdim
+    proj = hops.matmul(h, w["w_proj"])          # q | k | v | g
+    z = torch.addmm(w["b_a2"], hops.rowdot(h, w["w_a1"]), w["w_a2t"])  # float32 decay logits [T, H D]
+    decay = hops.decay_pow(z, 1.0 / spec.tau)
+    o = hops.linear_scan(proj, 0, H * D, 2 * H * D, None, None, D ** -0.5, decay, None, meta.q_start, meta.pos0,
+                         meta.slots, cache.S[li], H, H, D, Dv)
+    return hops.matmul(hops.head_norm_gate(o, proj, 2 * H * D + H * Dv, w["norm"], model.cfg.norm_eps, True,
+                                           model.act_dtype), w["w_o"])
+
+
+def ff_glu(model, spec: GluFFSpec, w: dict, h):
+    return hops.matmul(hops.glu(hops.matmul(h, w["w_gu"]), spec.limit, spec.slope, spec.shift, model.act_dtype),
+                       w["w_down"])
+
+
+def ff_moe_glu(model, spec: MoEGluSpec, w: dict, h):
+    idx, wt = hops.moe_route_topk(h, w["w_router"], w["b_router"], spec.top)
+    return hops.moe_glu_ffn(h, idx, wt, w["w_gu"], w["w_down"], spec.limit, spec.slope, spec.shift, model.act_dtype)
+
+
 def ff_dense(model, spec: DenseFFSpec, w: dict, h):
     return hops.matmul(hops.act_inplace(hops.matmul(h, w["w_up"]), spec.act), w["w_down"])
 
@@ -280,8 +498,12 @@ def ff_moe(model, spec: MoEFFSpec, w: dict, h):
     return hops.moe_ffn(h, idx, wt, w["w_up"], w["w_down"], spec.act, model.act_dtype)
 
 
-MIXERS = {"mlstm": (mix_mlstm, pack_mlstm), "latent_attention": (mix_latent_attention, pack_latent)}
-FEED_FORWARDS = {"dense": (ff_dense, pack_dense), "moe": (ff_moe, pack_moe)}
+MIXERS = {"mlstm": (mix_mlstm, pack_mlstm), "latent_attention": (mix_latent_attention, pack_latent),
+          "window_attention": (mix_window_attention, pack_window_attention),
+          "delta_rule": (mix_delta_rule, pack_delta_rule), "gla": (mix_gla, pack_gla)}
+FEED_FORWARDS = {"dense": (ff_dense, pack_dense), "moe": (ff_moe, pack_moe), "glu": (ff_glu, pack_glu),
+                 "moe_glu": (ff_moe_glu, pack_moe_glu)}
+RECURRENT_MIXERS = ("mlstm", "delta_rule", "gla")
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -308,9 +530,13 @@ class HybridDecoder:
         self.sequence_parallel = False
         self.decode_overlap_rows = 0
         P = max_position or cfg.max_position
-        self.rope = {li: rope_cos_sin(l.mixer.rope_base, l.mixer.rope_dims, P, self.device)
-                     for li, l in enumerate(cfg.layers) if l.mixer.kind == "latent_attention"}
-        self.recurrent = any(l.mixer.kind == "mlstm" for l in cfg.layers)
+        self.rope = {li: rope_cos_sin(l.mixer.rope_base, l.mixer.rope_dims, P, self.device,
+                                      getattr(l.mixer, "rope_scaling", None))
+                     for li, l in enumerate(cfg.layers)
+                     if l.mixer.kind in ("latent_attention", "window_attention") and l.mixer.rope_dims}
+        self.recurrent = any(l.mixer.kind in RECURRENT_MIXERS for l in cfg.layers)
+        if cfg.residual not in ("out_norm", "post_norm"):
+            raise ValueError(f"unknown residual rule {cfg.residual!r}")
 
     # ---- what the engine calls --------------------------------------------------------------------------------
     def make_cache(self, num_blocks: int, block_size: int, slots: int, kv_dtype: str = "bf16", k_scale: float = 1.0,
@@ -373,16 +599,25 @@ class HybridDecoder:
         x, h = hops.embed_rows(meta.ids, w.embed, at)
         for li, (spec, lw) in enumerate(zip(cfg.layers, w.layers)):
             y = MIXERS[spec.mixer.kind][0](self, li, spec.mixer, lw.mix, h, meta, cache)
-            h = hops.add_layer_norm(y, x, lw.norm1, cfg.norm_eps, at)
+            h = self._join(y, x, lw.norm1)
             if spec.ff is not None:
                 y = FEED_FORWARDS[spec.ff.kind][0](self, spec.ff, lw.ff, h)
-                h = hops.add_layer_norm(y, x, lw.norm2, cfg.norm_eps, at)
+                h = self._join(y, x, lw.norm2)
             if self.layer_tap is not None:
                 self.layer_tap(li, x)
         xs = x.index_select(0, meta.last_idx)
-        logits = hops.matmul(hops.layer_norm(xs, w.final_norm, cfg.norm_eps, at), w.head).float()
+        final = hops.rms_norm if cfg.residual == "post_norm" else hops.layer_norm
+        logits = hops.matmul(final(xs, w.final_norm, cfg.norm_eps, at), w.head).float()
         if cfg.logit_scale != 1.0:
             logits = logits * cfg.logit_scale
         return logits if logits.dtype == logits_dtype else logits.to(logits_dtype)
+
+    def _join(self, y, x, w):
+        """The residual rule: folds the sublayer output y into the float32 stream x (in place) and returns the
+        stream in the activation dtype for the next sublayer."""
+        cfg = self.cfg
+        if cfg.residual == "post_norm":
+            return hops.scale_add_rms_norm(y, x, w, cfg.residual_alpha, cfg.norm_eps, self.act_dtype)
+        return hops.add_layer_norm(y, x, w, cfg.norm_eps, self.act_dtype)
 
     layer_tap = None  # debugging hook: called with (layer index, residual stream) after every layer

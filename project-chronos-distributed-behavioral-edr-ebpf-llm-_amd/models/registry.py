@@ -125,5 +125,28 @@ def _zokunex_presets():
     return list(zokunex.PRESETS)
 
 
+def _kalesun_build(name, device, tp, seed, is_path, max_position, weight_dtype, dtype):
+    from . import kalesun
+
+    if tp.world > 1:
+        raise NotImplementedError("Kalesun runs on full-weight ranks (data-parallel replicas)")
+    if weight_dtype != "bf16":
+        raise NotImplementedError("Kalesun weights are served in the activation dtype (no fp8 projections)")
+    return kalesun.build(name, device, seed, DTYPES[dtype], max_position)
+
+
+def _kalesun_is_checkpoint(path: str) -> bool:
+    from . import kalesun
+
+    return kalesun.is_checkpoint(path)
+
+
+def _kalesun_presets():
+    from . import kalesun
+
+    return list(kalesun.PRESETS)
+
+
+register(Family("kalesun", _kalesun_presets, _kalesun_is_checkpoint, _kalesun_build, ("bf16", "fp32")))
 register(Family("zokunex", _zokunex_presets, _zokunex_is_checkpoint, _zokunex_build, ("bf16", "fp32")))
 register(Family("llama", _llama_presets, _llama_is_checkpoint, _llama_build, ("bf16",)))

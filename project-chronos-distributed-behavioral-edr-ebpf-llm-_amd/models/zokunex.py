@@ -175,6 +175,11 @@ class _SafetensorsDir:
             raise KeyError(f"checkpoint has no tensor {name!r}")
         return self._where[name].get_tensor(name)
 
+    def shape(self, name) -> tuple:
+        if name not in self._where:
+            raise KeyError(f"checkpoint has no tensor {name!r}")
+        return tuple(self._where[name].get_slice(name).get_shape())
+
 
 def is_checkpoint(path: str) -> bool:
     cj = os.path.join(path, "config.json")

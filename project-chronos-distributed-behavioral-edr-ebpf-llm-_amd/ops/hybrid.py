@@ -16,7 +16,7 @@ import os
 import torch
 
 from . import hybrid_ref as ref
-from .hybrid_ref import ACT_GELU, ACT_RELU2  # noqa: F401
+from .hybrid_ref import ACT_GELU, ACT_GLU, ACT_RELU2  # noqa: F401
 
 _REF_ON_GPU = os.environ.get("CHRONOS_HYBRID_REF", "0") not in ("", "0")
 
@@ -129,3 +129,93 @@ def moe_ffn(h, idx, wt, w_up, w_down, act: int, act_dtype):
     if _gpu(h):
         return _k().hy_moe_ffn(h, idx, wt, w_up, w_down, act)
     return ref.moe_ffn(h, idx, wt, w_up, w_down, act, act_dtype)
+
+
+# ---- post-norm residual stream, clamped GLU, windowed attention with sinks, linear-state recurrences ---------------
+
+
+def rms_norm(x, w, eps: float, act_dtype):
+    if _gpu(x):
+        return _k().hy_rms_norm(x, w, eps, _f32(act_dtype))
+    return ref.rms_norm(x, w, eps, act_dtype)
+
+
+def scale_add_rms_norm(y, x, w, alpha: float, eps: float, act_dtype):
+    """x (float32 residual, in place) <- rms_norm(alpha * x + y) * w; returns the updated rows in the activation
+    dtype (x itself when that is float32)."""
+    if _gpu(x):
+        h = _k().hy_scale_add_rms_norm(y, x, w, alpha, eps, _f32(act_dtype))
+        return x if _f32(act_dtype) else h
+    return ref.scale_add_rms_norm(y, x, w, alpha, eps, act_dtype)
+
+
+def glu(gu, limit: float, slope: float, shift: float, act_dtype):
+    if _gpu(gu):
+        return _k().hy_glu(gu, limit, slope, shift)
+    return ref.glu(gu, limit, slope, shift, act_dtype)
+
+
+def window_prep(qkv, H: int, G: int, D: int, Dv: int, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm,
+                eps: float, cos_sin, dims: int, kc, vc, emit_v: bool):
+    if _gpu(qkv):
+        v = _k().hy_window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin,
+                                dims, kc, vc, emit_v)
+        return v if emit_v else None
+    return ref.window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin,
+                           dims, kc, vc, emit_v)
+
+
+def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale: float, window: int, keep_first: int,
+                     H: int, act_dtype, max_q: int):
+    """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid)."""
+    if _gpu(qkv):
+        return _k().hy_window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first,
+                                        H, max_q)
+    return ref.window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H,
+                                act_dtype)
+
+
+def short_conv(x, w, q_start, pos0, slots, hist, silu: bool = True):
+    if _gpu(x):
+        return _k().hy_short_conv(x, w, q_start, pos0, slots, hist, silu)
+    return ref.short_conv(x, w, q_start, pos0, slots, hist, silu)
+
+
+def delta_prep(y, ab, a_log, HK: int, H: int, D: int, q_mul: float):
+    if _gpu(y):
+        return _k().hy_delta_prep(y, ab, a_log, HK, H, D, q_mul)
+    return ref.delta_prep(y, ab, a_log, HK, H, D, q_mul)
+
+
+def decay_pow(z, inv_tau: float):
+    if _gpu(z):
+        _k().hy_decay_pow(z, inv_tau)
+        return z
+    return ref.decay_pow(z, inv_tau)
+
+
+def linear_scan(proj, q_off: int, k_off: int, v_off: int, qscale, kscale, q_mul: float, decay, beta, q_start, pos0,
+                slots, S, HK: int, H: int, D: int, Dv: int):
+    if _gpu(proj):
+        return _k().hy_linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots,
+                                   S, HK, H, D, Dv)
+    return ref.linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots, S, HK,
+                           H, D, Dv)
+
+
+def head_norm_gate(o, src, g_off: int, w, eps: float, silu_gate: bool, act_dtype):
+    if _gpu(o):
+        return _k().hy_head_norm_gate(o, src, g_off, w, eps, silu_gate, _f32(act_dtype))
+    return ref.head_norm_gate(o, src, g_off, w, eps, silu_gate, act_dtype)
+
+
+def moe_route_topk(h, w_router, bias, top: int):
+    if _gpu(h):
+        return _k().hy_moe_route_topk(h, w_router, bias, top)
+    return ref.moe_route_topk(h, w_router, bias, top)
+
+
+def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit: float, slope: float, shift: float, act_dtype):
+    if _gpu(h):
+        return _k().hy_moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift)
+    return ref.moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, act_dtype)

@@ -185,3 +185,216 @@ def moe_ffn(h, idx, wt, w_up, w_down, act, act_dtype):
     ident = (idl >= E).float() * wt
     out = out + ident.sum(-1, keepdim=True) * hf
     return out.to(act_dtype)
+
+
+# ---- post-norm residual stream, clamped GLU, windowed attention with sinks, linear-state recurrences ---------------
+
+ACT_GLU = 2  # gated unit: min(g, limit) * sigmoid(slope * g) * (clamp(u, +-limit) + shift)
+
+
+def rms_norm(x, w, eps, act_dtype):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(act_dtype)
+
+
+def scale_add_rms_norm(y, x, w, alpha, eps, act_dtype):
+    """x (float32, in place) <- rms_norm(alpha * x + y) * w; returns x in the activation dtype (x itself for
+    float32): the norm sits AFTER the residual sum and the stream itself is what the next sublayer reads."""
+    x.copy_(rms_norm(alpha * x + y.float(), w, eps, torch.float32))
+    return x if act_dtype == torch.float32 else x.to(act_dtype)
+
+
+def glu(gu, limit, slope, shift, act_dtype):
+    """gu [T, 2F]: gate columns then up columns -> [T, F]."""
+    F = gu.shape[1] // 2
+    g = gu[:, :F].float().clamp(max=limit)
+    u = gu[:, F:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(slope * g) * (u + shift)).to(act_dtype)
+
+
+def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin, dims, kc, vc,
+                emit_v):
+    """qkv [T, H D + G D + G Dv]: per-head RMS norm (weights q_norm / k_norm [D], float32 math) and rotation of the
+    query and key heads, queries in place; values mixed with ``v_first`` [T, G Dv] as (1 - lam) v + lam v_first when
+    given; keys and (mixed) values written to the paged caches kc [NB, BS, G, D], vc [NB, BS, G, Dv].  Returns the
+    values as read from the projection [T, G Dv] when ``emit_v`` (the source of later layers' mixing), else None."""
+    T = qkv.shape[0]
+    q = qkv[:, :H * D].view(T, H, D)
+    k = qkv[:, H * D:(H + G) * D].view(T, G, D)
+    v = qkv[:, (H + G) * D:].view(T, G, Dv)
+    out_v = v.reshape(T, G * Dv).clone() if emit_v else None
+
+    def norm_rot(x, w):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        return rotate_half_rows(xf, cos_sin, pos, dims) if dims else xf
+
+    qn = norm_rot(q, q_norm)
+    kn = norm_rot(k, k_norm)
+    vf = v.float()
+    if v_first is not None:
+        l = lam.float().reshape(())
+        vf = (1.0 - l) * vf + l * v_first.view(T, G, Dv).float()
+    bs = kc.shape[1]
+    blk = block_table[tok_seq.long(), (pos // bs).long()].long()
+    kc[blk, (pos % bs).long()] = kn.to(kc.dtype)
+    vc[blk, (pos % bs).long()] = vf.to(vc.dtype)
+    q.copy_(qn.to(q.dtype))
+    return out_v
+
+
+def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H, act_dtype):
+    """Causal softmax attention over a paged cache through a sliding window that also keeps a sequence's first
+    tokens: the query at position i sees key j <= i when i - j < window or j < keep_first (window 0: every j <= i).
+    ``sink`` f32 [H] or None: exp(sink_h) joins the softmax denominator (no key, no value).  ``gate`` f32 [T, H] or
+    None: head h's output times sigmoid(gate).  Queries are the first H D columns of qkv; query head h reads
+    key/value head h // (H / G).  Returns [T, H Dv]."""
+    T = qkv.shape[0]
+    G, D, Dv = kc.shape[2], kc.shape[3], vc.shape[3]
+    q = qkv[:, :H * D].view(T, H, D).float()
+    out = torch.zeros(T, H, Dv, dtype=torch.float32, device=qkv.device)
+    bs = kc.shape[1]
+    qs = q_start.tolist()
+    rep = H // G
+    for b in range(len(qs) - 1):
+        t0, t1 = qs[b], qs[b + 1]
+        if t1 <= t0:
+            continue
+        p = pos[t0:t1].long()
+        ctx = int(p.max()) + 1
+        nblk = (ctx + bs - 1) // bs
+        pages = block_table[b, :nblk].long()
+        keys = kc[pages].reshape(nblk * bs, G, D)[:ctx].float().repeat_interleave(rep, 1)
+        vals = vc[pages].reshape(nblk * bs, G, Dv)[:ctx].float().repeat_interleave(rep, 1)
+        sc = torch.einsum("thd,jhd->thj", q[t0:t1], keys) * scale
+        j = torch.arange(ctx, device=qkv.device)[None, :]
+        hidden = j > p[:, None]
+        if window:
+            hidden = hidden | ((p[:, None] - j >= window) & (j >= keep_first))
+        sc = sc.masked_fill(hidden[:, None, :], float("-inf"))
+        if sink is not None:
+            sc = torch.cat([sc, sink.float()[None, :, None].expand(t1 - t0, H, 1)], -1)
+        a = torch.softmax(sc, -1)[:, :, :ctx]
+        out[t0:t1] = torch.einsum("thj,jhv->thv", a, vals)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[:, :, None]
+    return out.reshape(T, H * Dv).to(act_dtype)
+
+
+def short_conv(x, w, q_start, pos0, slots, hist, silu):
+    """Causal per-channel convolution over time on a flattened token stream, on the first C columns of x [T, >= C];
+    w f32 [C, K] (the last column weighs the current token); hist [NS, K - 1, C]: every sequence's last K - 1 inputs
+    (oldest first), read when its range starts past position 0 (zeros otherwise) and updated in place.  Returns
+    [T, C] in x's dtype."""
+    C, K = w.shape
+    x = x[:, :C]
+    y = torch.empty_like(x)
+    qs, p0, sl = q_start.tolist(), pos0.tolist(), slots.tolist()
+    for b in range(len(sl)):
+        t0, t1 = qs[b], qs[b + 1]
+        if t1 <= t0:
+            continue
+        past = hist[sl[b]].clone() if p0[b] > 0 else torch.zeros(K - 1, C, dtype=x.dtype, device=x.device)
+        ext = torch.cat([past, x[t0:t1]], 0).float()
+        acc = torch.zeros(t1 - t0, C, dtype=torch.float32, device=x.device)
+        for i in range(K):
+            acc += ext[i:i + t1 - t0] * w[:, i].float()
+        if silu:
+            acc = acc * torch.sigmoid(acc)
+        y[t0:t1] = acc.to(x.dtype)
+        if K > 1:
+            hist[sl[b]] = ext[-(K - 1):].to(hist.dtype)
+    return y
+
+
+def delta_prep(y, ab, a_log, HK, H, D, q_mul):
+    """Per-token scalars of the gated delta rule.  y [T, >= 2 HK D]: q heads then k heads (after convolution and
+    activation); ab f32 [T, 2 H]: decay pre-activations (bias included) then write-strength pre-activations.
+    Returns float32 (qscale [T, HK] = q_mul / sqrt(|q|^2 + 1e-6), kscale [T, HK] = 1 / sqrt(|k|^2 + 1e-6),
+    decay [T, H] = exp(-exp(a_log) softplus(a)), beta [T, H] = sigmoid(b))."""
+    T = y.shape[0]
+    q = y[:, :HK * D].float().view(T, HK, D)
+    k = y[:, HK * D:2 * HK * D].float().view(T, HK, D)
+    qs = q_mul * torch.rsqrt(q.pow(2).sum(-1) + 1e-6)
+    ks = torch.rsqrt(k.pow(2).sum(-1) + 1e-6)
+    decay = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(ab[:, :H].float()))
+    return qs, ks, decay, torch.sigmoid(ab[:, H:2 * H].float())
+
+
+def decay_pow(z, inv_tau):
+    """z f32 (in place) <- sigmoid(z) ** inv_tau, through the logarithm."""
+    z.copy_(torch.exp(torch.nn.functional.logsigmoid(z) * inv_tau))
+    return z
+
+
+def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots, S, HK, H, D, Dv):
+    """Linear-state recurrence over a flattened token stream, per value head h (reading q/k head h // (H / HK)):
+
+        S <- decay * S                      decay f32 [T, H] (one per head) or [T, H, D] (one per key channel / row)
+        u  = v - S^T k, times beta          only when beta f32 [T, H] is given (the delta rule); else u = v
+        S <- S + k u^T;   o = S^T q
+
+    q, k, v are columns of proj [T, C] at q_off / k_off / v_off; q is multiplied by qscale [T, HK] (or by q_mul when
+    None) and k by kscale [T, HK] (when given), in float32.  S f32 [NS, H, D, Dv] by slot, in place; a range whose
+    first token sits at position 0 starts from zero.  Returns o f32 [T, H, Dv]."""
+    T = proj.shape[0]
+    out = torch.zeros(T, H, Dv, dtype=torch.float32, device=proj.device)
+    qs, p0, sl = q_start.tolist(), pos0.tolist(), slots.tolist()
+    pf = proj.float()
+    q = pf[:, q_off:q_off + HK * D].view(T, HK, D)
+    k = pf[:, k_off:k_off + HK * D].view(T, HK, D)
+    v = pf[:, v_off:v_off + H * Dv].view(T, H, Dv)
+    q = q * (qscale[:, :, None] if qscale is not None else q_mul)
+    if kscale is not None:
+        k = k * kscale[:, :, None]
+    rep = H // HK
+    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
+    dec = decay.view(T, H, -1, 1)  # [T, H, 1 | D, 1]
+    for b in range(len(sl)):
+        if qs[b + 1] <= qs[b]:
+            continue
+        Sb = torch.zeros_like(S[sl[b]]) if p0[b] == 0 else S[sl[b]].clone()
+        for t in range(qs[b], qs[b + 1]):
+            Sb = dec[t] * Sb
+            u = v[t]
+            if beta is not None:
+                u = beta[t][:, None] * (u - torch.einsum("hdv,hd->hv", Sb, k[t]))
+            Sb = Sb + k[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", Sb, q[t])
+        S[sl[b]] = Sb
+    return out
+
+
+def head_norm_gate(o, src, g_off, w, eps, silu_gate, act_dtype):
+    """Per-head unit RMS of o f32 [T, H, Dv], times w [H Dv], times sigmoid (or silu) of the gate columns
+    src[:, g_off : g_off + H Dv]."""
+    T, H, Dv = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+    g = src[:, g_off:g_off + H * Dv].float()
+    g = g * torch.sigmoid(g) if silu_gate else torch.sigmoid(g)
+    return (y.reshape(T, H * Dv) * w.float() * g).to(act_dtype)
+
+
+def moe_route_topk(h, w_router, bias, top):
+    """Router that picks the ``top`` largest logits (h W^T + bias, float32; ties: the lower index) and weighs them by
+    the softmax over the chosen logits only.  Returns (idx int32 [T, top], weight f32 [T, top])."""
+    z = rowdot(h, w_router, bias)
+    val, idx = torch.topk(z, top, dim=-1)
+    return idx.to(torch.int32), torch.softmax(val, -1)
+
+
+def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, act_dtype):
+    """Weighted sum of each token's chosen gated experts.  w_gu [E, 2F, d]: gate rows then up rows; w_down
+    [E, d, F]."""
+    E = w_gu.shape[0]
+    hf = h.float()
+    out = torch.zeros_like(hf)
+    idl = idx.long()
+    for e in range(E):
+        tok, kk = torch.nonzero(idl == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        gu = hf[tok].to(act_dtype) @ w_gu[e].t().to(act_dtype)
+        y = (glu(gu, limit, slope, shift, act_dtype) @ w_down[e].t().to(act_dtype)).float()
+        out.index_add_(0, tok, y * wt[tok, kk][:, None])
+    return out.to(act_dtype)
