@@ -36,6 +36,29 @@ void launch_hy_moe_ffn_token(const void*, const int32_t*, const float*, const vo
 int hy_moe_max_tiles(int, int);
 void launch_hy_moe_grouped(const uint16_t*, const int32_t*, const float*, const uint16_t*, const uint16_t*, uint16_t*,
                            int32_t*, uint16_t*, uint16_t*, int, int, int, int, int, int, hipStream_t);
+void launch_hy_rms_norm(const void*, float*, const float*, void*, bool, int, int, float, float, hipStream_t);
+void launch_hy_glu(const void*, void*, int64_t, int, float, float, float, bool, hipStream_t);
+void launch_hy_decay_pow(float*, int64_t, float, hipStream_t);
+void launch_hy_head_norm_gate(const float*, const void*, int, int, const float*, void*, int, int, int, float, bool, bool,
+                              hipStream_t);
+void launch_hy_window_prep(void*, int, int, int, int, int, const void*, const float*, const int32_t*, const int32_t*,
+                           const int32_t*, int, const float*, const float*, float, const float*, int, void*, void*, int,
+                           void*, int, bool, hipStream_t);
+size_t hy_window_attention_lds(int, int, bool);
+void launch_hy_window_attention(const void*, int, const void*, const void*, const int32_t*, int, const int32_t*,
+                                const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
+                                int, int, bool, hipStream_t);
+void launch_hy_short_conv(const void*, int, const float*, const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                          void*, void*, int, int, int, int, bool, bool, hipStream_t);
+void launch_hy_delta_prep(const void*, int, const float*, const float*, float*, float*, float*, float*, int, int, int, int,
+                          float, bool, hipStream_t);
+bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const float*, float, const float*, bool,
+                           const float*, const int32_t*, const int32_t*, const int32_t*, float*, float*, int, int, int, int,
+                           int, bool, hipStream_t);
+void launch_hy_moe_route_topk(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
+                              hipStream_t);
+void launch_hy_moe_glu_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
+                             int, int, float, float, float, bool, hipStream_t);
 }  // namespace chronos
 
 namespace {
@@ -258,6 +281,222 @@ Tensor hy_moe_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, const Te
     return out;
 }
 
+Tensor hy_rms_norm(const Tensor& x, const Tensor& w, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "rms_norm: float32 rows");
+    flt(w, "rms_norm: float32 weight");
+    need(x.dim() == 2 && w.numel() == x.size(1), "rms_norm: weight size");
+    auto h = at::empty_like(x, x.options().dtype(out_f32 ? at::kFloat : at::kBFloat16));
+    chronos::launch_hy_rms_norm(nullptr, const_cast<float*>(x.data_ptr<float>()), w.data_ptr<float>(), h.data_ptr(),
+                                out_f32, (int)x.size(0), (int)x.size(1), 1.f, (float)eps, stream());
+    return h;
+}
+
+Tensor hy_scale_add_rms_norm(const Tensor& y, Tensor& x, const Tensor& w, double alpha, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "scale_add_rms_norm: float32 residual");
+    flt(w, "scale_add_rms_norm: float32 weight");
+    need(is_act(y) && y.is_contiguous() && y.dim() == 2 && y.sizes() == x.sizes(), "scale_add_rms_norm: y shape");
+    need(f32(y) == out_f32, "scale_add_rms_norm: y must be in the activation dtype");
+    need(w.numel() == x.size(1), "scale_add_rms_norm: weight size");
+    Tensor h = out_f32 ? at::empty({0}, x.options()) : at::empty_like(x, x.options().dtype(at::kBFloat16));
+    chronos::launch_hy_rms_norm(y.data_ptr(), x.data_ptr<float>(), w.data_ptr<float>(), out_f32 ? nullptr : h.data_ptr(),
+                                out_f32, (int)x.size(0), (int)x.size(1), (float)alpha, (float)eps, stream());
+    return h;
+}
+
+Tensor hy_glu(const Tensor& gu, double limit, double slope, double shift) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(gu.device());
+    need(is_act(gu) && gu.dim() == 2 && gu.is_contiguous() && gu.size(1) % 2 == 0, "glu: [T, 2F] activation tensor");
+    auto y = at::empty({gu.size(0), gu.size(1) / 2}, gu.options());
+    chronos::launch_hy_glu(gu.data_ptr(), y.data_ptr(), gu.size(0), (int)(gu.size(1) / 2), (float)limit, (float)slope,
+                           (float)shift, f32(gu), stream());
+    return y;
+}
+
+void hy_decay_pow(Tensor& z, double p) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(z.device());
+    flt(z, "decay_pow: float32 contiguous logits");
+    chronos::launch_hy_decay_pow(z.data_ptr<float>(), z.numel(), (float)p, stream());
+}
+
+Tensor hy_head_norm_gate(const Tensor& o, const Tensor& src, int64_t g_off, const Tensor& w, double eps, bool silu_gate,
+                         bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+    flt(o, "head_norm_gate: float32 read-out");
+    flt(w, "head_norm_gate: float32 weight");
+    need(o.dim() == 3 && is_act(src) && src.dim() == 2 && src.is_contiguous() && src.size(0) == o.size(0), "head_norm_gate: shapes");
+    const int64_t T = o.size(0), H = o.size(1), Dv = o.size(2);
+    need(f32(src) == out_f32 && g_off >= 0 && g_off + H * Dv <= src.size(1) && w.numel() == H * Dv, "head_norm_gate: gate columns / weight");
+    auto y = at::empty({T, H * Dv}, src.options());
+    chronos::launch_hy_head_norm_gate(o.data_ptr<float>(), src.data_ptr(), (int)src.size(1), (int)g_off, w.data_ptr<float>(),
+                                      y.data_ptr(), (int)T, (int)H, (int)Dv, (float)eps, silu_gate, out_f32, stream());
+    return y;
+}
+
+Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, const c10::optional<Tensor>& v_first,
+                      const c10::optional<Tensor>& lam, const Tensor& pos, const Tensor& tok_seq, const Tensor& block_table,
+                      const Tensor& q_norm, const Tensor& k_norm, double eps, const c10::optional<Tensor>& cos_sin,
+                      int64_t dims, Tensor& kc, Tensor& vc, bool emit_v) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
+    same_act(qkv, kc, "window_prep: the caches hold the activation dtype");
+    same_act(qkv, vc, "window_prep: the caches hold the activation dtype");
+    need(qkv.dim() == 2 && qkv.is_contiguous() && kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous(), "window_prep: layouts");
+    const int64_t T = qkv.size(0);
+    need(H >= 1 && G >= 1 && H % G == 0 && D >= 1 && Dv >= 1 && qkv.size(1) == (H + G) * D + G * Dv, "window_prep: qkv width");
+    need(kc.size(2) == G && kc.size(3) == D && vc.size(2) == G && vc.size(3) == Dv && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "window_prep: cache shapes");
+    i32(pos, "window_prep: pos"); i32(tok_seq, "window_prep: tok_seq"); i32(block_table, "window_prep: block_table");
+    need(pos.numel() == T && tok_seq.numel() == T && block_table.dim() == 2, "window_prep: per-token metadata");
+    flt(q_norm, "window_prep: float32 norm weight"); flt(k_norm, "window_prep: float32 norm weight");
+    need(q_norm.numel() == D && k_norm.numel() == D, "window_prep: norm weights [D]");
+    need(dims >= 0 && dims % 2 == 0 && dims <= D, "window_prep: rotated columns");
+    if (dims > 0) {
+        need(cos_sin.has_value(), "window_prep: rotation needs the cos/sin table");
+        flt(*cos_sin, "window_prep: float32 cos/sin table");
+        need(cos_sin->dim() == 2 && cos_sin->size(1) == dims, "window_prep: table width");
+    }
+    if (v_first) {
+        same_act(qkv, *v_first, "window_prep: v_first in the activation dtype");
+        need(v_first->is_contiguous() && v_first->numel() == T * G * Dv, "window_prep: v_first [T, G Dv]");
+        need(lam.has_value(), "window_prep: mixing needs its weight");
+        flt(*lam, "window_prep: float32 mixing weight");
+        need(lam->numel() == 1, "window_prep: one mixing weight");
+    }
+    Tensor v_out = emit_v ? at::empty({T, G * Dv}, qkv.options()) : at::empty({0}, qkv.options());
+    chronos::launch_hy_window_prep(qkv.data_ptr(), (int)qkv.size(1), (int)H, (int)G, (int)D, (int)Dv,
+                                   v_first ? v_first->data_ptr() : nullptr, v_first ? lam->data_ptr<float>() : nullptr,
+                                   pos.data_ptr<int32_t>(), tok_seq.data_ptr<int32_t>(), block_table.data_ptr<int32_t>(),
+                                   (int)block_table.size(1), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), (float)eps,
+                                   dims > 0 ? cos_sin->data_ptr<float>() : nullptr, (int)dims, kc.data_ptr(), vc.data_ptr(),
+                                   (int)kc.size(1), emit_v ? v_out.data_ptr() : nullptr, (int)T, f32(qkv), stream());
+    return v_out;
+}
+
+Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc, const Tensor& block_table,
+                           const Tensor& q_start, const Tensor& pos, const c10::optional<Tensor>& sink,
+                           const c10::optional<Tensor>& gate, double scale, int64_t window, int64_t keep, int64_t H,
+                           int64_t max_q) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
+    same_act(qkv, kc, "window_attention: queries and caches in one activation dtype");
+    same_act(qkv, vc, "window_attention: queries and caches in one activation dtype");
+    need(qkv.dim() == 2 && qkv.is_contiguous() && kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous(), "window_attention: layouts");
+    const int64_t T = qkv.size(0), G = kc.size(2), D = kc.size(3), Dv = vc.size(3);
+    need(H >= 1 && H % G == 0 && qkv.size(1) >= H * D && vc.size(2) == G && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "window_attention: shapes");
+    need(H / G <= 64 && Dv <= 256, "window_attention: at most 64 query heads per key/value head and 256 value columns");
+    need(chronos::hy_window_attention_lds((int)D, (int)Dv, f32(qkv)) <= 160 * 1024, "window_attention: a key tile and 64 query rows must fit the LDS");
+    i32(block_table, "window_attention: block_table"); i32(q_start, "window_attention: q_start"); i32(pos, "window_attention: pos");
+    const int64_t B = q_start.numel() - 1;
+    need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T && window >= 0 && keep >= 0, "window_attention: metadata");
+    if (sink) { flt(*sink, "window_attention: float32 sinks"); need(sink->numel() == H, "window_attention: sink [H]"); }
+    if (gate) { flt(*gate, "window_attention: float32 gate"); need(gate->numel() == T * H, "window_attention: gate [T, H]"); }
+    auto out = at::empty({T, H * Dv}, qkv.options());
+    if (T == 0 || B <= 0) return out;
+    chronos::launch_hy_window_attention(qkv.data_ptr(), (int)qkv.size(1), kc.data_ptr(), vc.data_ptr(),
+                                        block_table.data_ptr<int32_t>(), (int)block_table.size(1),
+                                        q_start.data_ptr<int32_t>(), pos.data_ptr<int32_t>(),
+                                        sink ? sink->data_ptr<float>() : nullptr, gate ? gate->data_ptr<float>() : nullptr,
+                                        out.data_ptr(), (int)B, (int)std::max<int64_t>(1, max_q), (int)H, (int)G, (int)D,
+                                        (int)Dv, (int)kc.size(1), (float)scale, (int)window, (int)keep, f32(qkv), stream());
+    return out;
+}
+
+Tensor hy_short_conv(const Tensor& x, const Tensor& w, const Tensor& tok_seq, const Tensor& q_start, const Tensor& pos0,
+                     const Tensor& slots, Tensor& hist, bool silu) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    same_act(x, hist, "short_conv: the history holds the activation dtype");
+    flt(w, "short_conv: float32 taps");
+    need(x.dim() == 2 && x.is_contiguous() && w.dim() == 2 && hist.dim() == 3 && hist.is_contiguous(), "short_conv: layouts");
+    const int64_t T = x.size(0), C = w.size(0), K = w.size(1), B = slots.numel();
+    need(C <= x.size(1) && K >= 1 && hist.size(1) == K - 1 && hist.size(2) == C, "short_conv: channels / taps / history");
+    i32(tok_seq, "short_conv: tok_seq"); i32(q_start, "short_conv: q_start"); i32(pos0, "short_conv: pos0"); i32(slots, "short_conv: slots");
+    need(tok_seq.numel() == T && q_start.numel() == B + 1 && pos0.numel() == B, "short_conv: metadata");
+    auto y = at::empty({T, C}, x.options());
+    chronos::launch_hy_short_conv(x.data_ptr(), (int)x.size(1), w.data_ptr<float>(), tok_seq.data_ptr<int32_t>(),
+                                  q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(), slots.data_ptr<int32_t>(),
+                                  hist.data_ptr(), y.data_ptr(), (int)T, (int)B, (int)C, (int)K, silu, f32(x), stream());
+    return y;
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> hy_delta_prep(const Tensor& y, const Tensor& ab, const Tensor& a_log, int64_t HK,
+                                                         int64_t H, int64_t D, double q_mul) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(y.device());
+    need(is_act(y) && y.dim() == 2 && y.is_contiguous() && y.size(1) >= 2 * HK * D, "delta_prep: y [T, >= 2 HK D]");
+    flt(ab, "delta_prep: float32 pre-activations"); flt(a_log, "delta_prep: float32 A_log");
+    const int64_t T = y.size(0);
+    need(ab.numel() == T * 2 * H && a_log.numel() == H, "delta_prep: ab [T, 2H], a_log [H]");
+    auto fo = y.options().dtype(at::kFloat);
+    auto qs = at::empty({T, HK}, fo), ks = at::empty({T, HK}, fo), dc = at::empty({T, H}, fo), bt = at::empty({T, H}, fo);
+    chronos::launch_hy_delta_prep(y.data_ptr(), (int)y.size(1), ab.data_ptr<float>(), a_log.data_ptr<float>(),
+                                  qs.data_ptr<float>(), ks.data_ptr<float>(), dc.data_ptr<float>(), bt.data_ptr<float>(),
+                                  (int)T, (int)HK, (int)H, (int)D, (float)q_mul, f32(y), stream());
+    return {qs, ks, dc, bt};
+}
+
+Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t v_off, const c10::optional<Tensor>& qscale,
+                      const c10::optional<Tensor>& kscale, double q_mul, const Tensor& decay,
+                      const c10::optional<Tensor>& beta, const Tensor& q_start, const Tensor& pos0, const Tensor& slots,
+                      Tensor& S, int64_t HK, int64_t H, int64_t D, int64_t Dv) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+    need(is_act(proj) && proj.dim() == 2 && proj.is_contiguous(), "linear_scan: proj [T, C]");
+    const int64_t T = proj.size(0), C = proj.size(1), B = slots.numel();
+    need(HK >= 1 && H % HK == 0 && D >= 1 && Dv >= 1, "linear_scan: head counts");
+    need(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + HK * D <= C && k_off + HK * D <= C && v_off + H * Dv <= C, "linear_scan: column ranges");
+    flt(decay, "linear_scan: float32 decay");
+    const bool chd = decay.numel() == T * H * D && D > 1;
+    need(chd || decay.numel() == T * H, "linear_scan: decay [T, H] or [T, H, D]");
+    if (qscale) { flt(*qscale, "linear_scan: qscale"); need(qscale->numel() == T * HK, "linear_scan: qscale [T, HK]"); }
+    if (kscale) { flt(*kscale, "linear_scan: kscale"); need(kscale->numel() == T * HK, "linear_scan: kscale [T, HK]"); }
+    if (beta) { flt(*beta, "linear_scan: beta"); need(beta->numel() == T * H, "linear_scan: beta [T, H]"); }
+    i32(q_start, "linear_scan: q_start"); i32(pos0, "linear_scan: pos0"); i32(slots, "linear_scan: slots");
+    need(q_start.numel() == B + 1 && pos0.numel() == B, "linear_scan: q_start [B+1], pos0 [B], slots [B]");
+    flt(S, "linear_scan: S");
+    need(S.dim() == 4 && S.size(1) == H && S.size(2) == D && S.size(3) == Dv, "linear_scan: S [NS, H, D, Dv]");
+    auto o = at::empty({T, H, Dv}, proj.options().dtype(at::kFloat));
+    if (T == 0) return o;
+    const bool ok = chronos::launch_hy_linear_scan(
+        proj.data_ptr(), (int)C, (int)q_off, (int)k_off, (int)v_off, qscale ? qscale->data_ptr<float>() : nullptr,
+        kscale ? kscale->data_ptr<float>() : nullptr, (float)q_mul, decay.data_ptr<float>(), chd,
+        beta ? beta->data_ptr<float>() : nullptr, q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(),
+        slots.data_ptr<int32_t>(), S.data_ptr<float>(), o.data_ptr<float>(), (int)B, (int)HK, (int)H, (int)D, (int)Dv,
+        f32(proj), stream());
+    TORCH_CHECK(ok, "chronos hybrid op: linear_scan keeps a state column in registers, D <= 256 (got ", D, ")");
+    return o;
+}
+
+std::tuple<Tensor, Tensor> hy_moe_route_topk(const Tensor& h, const Tensor& w, const Tensor& bias, int64_t top) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w, "moe_route_topk: h and router in one activation dtype");
+    need(h.dim() == 2 && w.dim() == 2 && h.is_contiguous() && w.is_contiguous() && h.size(1) == w.size(1), "moe_route_topk: shapes");
+    flt(bias, "moe_route_topk: float32 bias");
+    const int64_t N = w.size(0);
+    need(bias.numel() == N && N <= 256 && top >= 1 && top <= N && top <= 64, "moe_route_topk: 1 <= top <= min(outputs, 64), outputs <= 256");
+    auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
+    auto wt = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
+    auto z = at::empty({h.size(0), N}, h.options().dtype(at::kFloat));
+    chronos::launch_hy_moe_route_topk(h.data_ptr(), w.data_ptr(), bias.data_ptr<float>(), z.data_ptr<float>(),
+                                      idx.data_ptr<int32_t>(), wt.data_ptr<float>(), (int)h.size(0), (int)h.size(1), (int)N,
+                                      (int)top, f32(h), stream());
+    return {idx, wt};
+}
+
+Tensor hy_moe_glu_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, const Tensor& w_gu, const Tensor& w_down,
+                      double limit, double slope, double shift) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w_gu, "moe_glu_ffn: h and experts in one activation dtype");
+    same_act(h, w_down, "moe_glu_ffn: h and experts in one activation dtype");
+    need(h.dim() == 2 && h.is_contiguous() && w_gu.dim() == 3 && w_down.dim() == 3 && w_gu.is_contiguous() && w_down.is_contiguous(), "moe_glu_ffn: layouts");
+    const int64_t T = h.size(0), d = h.size(1), E = w_gu.size(0), F = w_down.size(2);
+    need(w_gu.size(1) == 2 * F && w_gu.size(2) == d && w_down.size(0) == E && w_down.size(1) == d, "moe_glu_ffn: expert shapes");
+    i32(idx, "moe_glu_ffn: idx"); flt(wt, "moe_glu_ffn: weights");
+    need(idx.dim() == 2 && idx.size(0) == T && wt.sizes() == idx.sizes(), "moe_glu_ffn: idx / weights [T, top]");
+    need((2 * d + 2 * F) * 4 <= 160 * 1024, "moe_glu_ffn: a token's rows must fit the LDS");
+    auto out = at::empty_like(h);
+    chronos::launch_hy_moe_glu_token(h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(), w_gu.data_ptr(),
+                                     w_down.data_ptr(), out.data_ptr(), (int)T, (int)d, (int)F, (int)E, (int)idx.size(1),
+                                     (float)limit, (float)slope, (float)shift, f32(h), stream());
+    return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(chronos, m) {
@@ -276,6 +515,25 @@ TORCH_LIBRARY_FRAGMENT(chronos, m) {
           "float scale, int rank, int max_q) -> Tensor");
     m.def("hy_moe_route(Tensor h, Tensor w, Tensor corr, int top) -> (Tensor, Tensor)");
     m.def("hy_moe_ffn(Tensor h, Tensor idx, Tensor wt, Tensor w_up, Tensor w_down, int act) -> Tensor");
+    m.def("hy_rms_norm(Tensor x, Tensor w, float eps, bool out_f32) -> Tensor");
+    m.def("hy_scale_add_rms_norm(Tensor y, Tensor(a!) x, Tensor w, float alpha, float eps, bool out_f32) -> Tensor");
+    m.def("hy_glu(Tensor gu, float limit, float slope, float shift) -> Tensor");
+    m.def("hy_decay_pow(Tensor(a!) z, float p) -> ()");
+    m.def("hy_head_norm_gate(Tensor o, Tensor src, int g_off, Tensor w, float eps, bool silu_gate, bool out_f32) -> Tensor");
+    m.def("hy_window_prep(Tensor(a!) qkv, int H, int G, int D, int Dv, Tensor? v_first, Tensor? lam, Tensor pos, "
+          "Tensor tok_seq, Tensor block_table, Tensor q_norm, Tensor k_norm, float eps, Tensor? cos_sin, int dims, "
+          "Tensor(b!) kc, Tensor(c!) vc, bool emit_v) -> Tensor");
+    m.def("hy_window_attention(Tensor qkv, Tensor kc, Tensor vc, Tensor block_table, Tensor q_start, Tensor pos, "
+          "Tensor? sink, Tensor? gate, float scale, int window, int keep, int H, int max_q) -> Tensor");
+    m.def("hy_short_conv(Tensor x, Tensor w, Tensor tok_seq, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) hist, "
+          "bool silu) -> Tensor");
+    m.def("hy_delta_prep(Tensor y, Tensor ab, Tensor a_log, int HK, int H, int D, float q_mul) -> (Tensor, Tensor, Tensor, Tensor)");
+    m.def("hy_linear_scan(Tensor proj, int q_off, int k_off, int v_off, Tensor? qscale, Tensor? kscale, float q_mul, "
+          "Tensor decay, Tensor? beta, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) S, int HK, int H, int D, "
+          "int Dv) -> Tensor");
+    m.def("hy_moe_route_topk(Tensor h, Tensor w, Tensor bias, int top) -> (Tensor, Tensor)");
+    m.def("hy_moe_glu_ffn(Tensor h, Tensor idx, Tensor wt, Tensor w_gu, Tensor w_down, float limit, float slope, "
+          "float shift) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(chronos, CUDA, m) {
@@ -291,4 +549,16 @@ TORCH_LIBRARY_IMPL(chronos, CUDA, m) {
     m.impl("hy_latent_attention", &hy_latent_attention);
     m.impl("hy_moe_route", &hy_moe_route);
     m.impl("hy_moe_ffn", &hy_moe_ffn);
+    m.impl("hy_rms_norm", &hy_rms_norm);
+    m.impl("hy_scale_add_rms_norm", &hy_scale_add_rms_norm);
+    m.impl("hy_glu", &hy_glu);
+    m.impl("hy_decay_pow", &hy_decay_pow);
+    m.impl("hy_head_norm_gate", &hy_head_norm_gate);
+    m.impl("hy_window_prep", &hy_window_prep);
+    m.impl("hy_window_attention", &hy_window_attention);
+    m.impl("hy_short_conv", &hy_short_conv);
+    m.impl("hy_delta_prep", &hy_delta_prep);
+    m.impl("hy_linear_scan", &hy_linear_scan);
+    m.impl("hy_moe_route_topk", &hy_moe_route_topk);
+    m.impl("hy_moe_glu_ffn", &hy_moe_glu_ffn);
 }

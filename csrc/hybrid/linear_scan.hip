@@ -1,0 +1,284 @@
+// linear_scan.hip — recurrent mixers whose per-head state is a D x Dv matrix updated by rank-one writes: the gated
+// delta rule and gated linear attention, plus the short causal convolution and the per-token scalars that feed them.
+//
+//   short_conv    y[t, c] = act(sum_i w[c, i] x[t - (K-1) + i, c]) over each sequence's own tokens; inputs before the
+//                 step's first token come from the sequence's history rows (its last K-1 inputs, by state slot), or
+//                 are zero when the step starts at position 0.  A second launch then rewrites the history.
+//   delta_prep    per token: 1 / |q|, 1 / |k| per query/key head (float), decay = exp(-exp(A) softplus(a)) and
+//                 beta = sigmoid(b) per value head.
+//   linear_scan   per (sequence, value head, 64 value columns per wave): the state's column lives in registers (lane =
+//                 column, all D rows), tokens are staged 16 at a time in LDS (scaled q and k rows in float, the
+//                 decays, the values), and every token does
+//                     S <- decay * S;  u = v - S^T k (times beta; delta rule only, else u = v);  S <- S + k u^T;
+//                     o = S^T q
+//                 with no cross-lane traffic.  decay is one number per head or one per state row.  The same kernel
+//                 serves prompt portions of any length and decode rows (a range of one token); a range that starts at
+//                 position 0 starts from the zero state, so a reused slot needs no clearing.
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+template <typename T>
+__global__ void __launch_bounds__(256) short_conv_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                         const int32_t* __restrict__ tok_seq,
+                                                         const int32_t* __restrict__ q_start,
+                                                         const int32_t* __restrict__ pos0,
+                                                         const int32_t* __restrict__ slots, const T* __restrict__ hist,
+                                                         T* __restrict__ y, int C, int K, int silu) {
+    const int64_t t = blockIdx.x;
+    const int b = tok_seq[t];
+    const int t0 = q_start[b];
+    const bool past = pos0[b] > 0;
+    const T* hrow = hist + (int64_t)slots[b] * (K - 1) * C;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float acc = 0.f;
+        for (int i = 0; i < K; ++i) {
+            const int64_t s = t - (K - 1) + i;
+            float v = 0.f;
+            if (s >= t0) v = ld<T>(x + s * ldx + c);
+            else if (past) v = ld<T>(hrow + (int64_t)((K - 1) + (s - t0)) * C + c);
+            acc += w[c * K + i] * v;
+        }
+        if (silu) acc = acc * sigmoidf_(acc);
+        st<T>(y + t * C + c, acc);
+    }
+}
+
+// hist[slot][i] <- the input K-1-i tokens before the sequence's new end.  Entry i reads either this step's tokens or
+// an OLDER entry i + n (n >= 1 new tokens), so ascending i in place never reads what it has written.
+template <typename T>
+__global__ void __launch_bounds__(256) conv_hist_kernel(const T* __restrict__ x, int ldx,
+                                                        const int32_t* __restrict__ q_start,
+                                                        const int32_t* __restrict__ pos0,
+                                                        const int32_t* __restrict__ slots, T* __restrict__ hist, int C,
+                                                        int K) {
+    const int b = blockIdx.x;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    if (t1 <= t0) return;
+    const bool past = pos0[b] > 0;
+    T* hrow = hist + (int64_t)slots[b] * (K - 1) * C;
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+        for (int i = 0; i < K - 1; ++i) {
+            const int64_t s = (int64_t)t1 - (K - 1) + i;
+            T v;
+            if (s >= t0) v = x[s * ldx + c];
+            else if (past) v = hrow[(int64_t)((K - 1) + (s - t0)) * C + c];
+            else st<T>(&v, 0.f);
+            hrow[(int64_t)i * C + c] = v;
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) delta_prep_kernel(const T* __restrict__ y, int ldy, const float* __restrict__ ab,
+                                                         const float* __restrict__ a_log, float* __restrict__ qscale,
+                                                         float* __restrict__ kscale, float* __restrict__ decay,
+                                                         float* __restrict__ beta, int HK, int H, int D, float q_mul) {
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int j = wv; j < 2 * HK; j += 4) {
+        const T* row = y + t * ldy + (int64_t)j * D;
+        float ss = 0.f;
+        for (int i = lane; i < D; i += 64) {
+            const float v = ld<T>(row + i);
+            ss += v * v;
+        }
+        const float inv = 1.f / sqrtf(wave_sum(ss) + 1e-6f);
+        if (lane == 0) {
+            if (j < HK) qscale[t * HK + j] = inv * q_mul;
+            else kscale[t * HK + (j - HK)] = inv;
+        }
+    }
+    for (int h = threadIdx.x; h < H; h += 256) {
+        const float a = ab[t * 2 * H + h];
+        const float sp = a > 20.f ? a : log1pf(expf(a));
+        decay[t * H + h] = expf(-expf(a_log[h]) * sp);
+        beta[t * H + h] = sigmoidf_(ab[t * 2 * H + H + h]);
+    }
+}
+
+constexpr int kScanTC = 16;  // tokens per LDS stage
+
+// LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64 NW] | scalar decay [TC] | beta [TC]
+template <typename T, int DP, bool DELTA, bool CHD>
+__global__ void __launch_bounds__(256) linear_scan_kernel(
+        const T* __restrict__ proj, int ldp, int q_off, int k_off, int v_off, const float* __restrict__ qscale,
+        const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, const float* __restrict__ beta,
+        const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots,
+        float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv) {
+    extern __shared__ __attribute__((aligned(16))) float ls_smem[];
+    constexpr int TC = kScanTC;
+    const int NW = blockDim.x >> 6;
+    float* qs = ls_smem;
+    float* ks = qs + TC * DP;
+    float* ds = ks + TC * DP;
+    float* vs = ds + (CHD ? TC * DP : 0);
+    float* gs = vs + TC * 64 * NW;
+    float* bs = gs + TC;
+    const int b = blockIdx.x, hd = blockIdx.y;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    if (t1 <= t0) return;
+    const int hk = hd / (H / HK);
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int col0 = blockIdx.z * 64 * NW;
+    const int col = col0 + wv * 64 + lane;
+    const bool live = col < Dv;
+    float* Sp = S + (((int64_t)slots[b] * H + hd) * D) * Dv + col;
+    float st_[DP];
+    if (pos0[b] > 0 && live) {
+#pragma unroll
+        for (int r = 0; r < DP; ++r) st_[r] = r < D ? Sp[(int64_t)r * Dv] : 0.f;
+    } else {
+#pragma unroll
+        for (int r = 0; r < DP; ++r) st_[r] = 0.f;
+    }
+    for (int tb = t0; tb < t1; tb += TC) {
+        const int nt = min(TC, t1 - tb);
+        __syncthreads();  // the previous stage has been consumed
+        for (int i = threadIdx.x; i < nt * DP; i += blockDim.x) {
+            const int tt = i / DP, r = i % DP;
+            const int64_t t = tb + tt;
+            float qv = 0.f, kv = 0.f;
+            if (r < D) {
+                qv = ld<T>(proj + t * ldp + q_off + hk * D + r) * (qscale != nullptr ? qscale[t * HK + hk] : q_mul);
+                kv = ld<T>(proj + t * ldp + k_off + hk * D + r) * (kscale != nullptr ? kscale[t * HK + hk] : 1.f);
+            }
+            qs[i] = qv;
+            ks[i] = kv;
+            if constexpr (CHD) ds[i] = r < D ? decay[(t * H + hd) * D + r] : 0.f;
+        }
+        for (int i = threadIdx.x; i < nt * 64 * NW; i += blockDim.x) {
+            const int tt = i / (64 * NW), c = col0 + i % (64 * NW);
+            vs[i] = c < Dv ? ld<T>(proj + (int64_t)(tb + tt) * ldp + v_off + hd * Dv + c) : 0.f;
+        }
+        if (threadIdx.x < nt) {
+            if constexpr (!CHD) gs[threadIdx.x] = decay[(int64_t)(tb + threadIdx.x) * H + hd];
+            if constexpr (DELTA) bs[threadIdx.x] = beta[(int64_t)(tb + threadIdx.x) * H + hd];
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const f32x4* q4 = reinterpret_cast<const f32x4*>(qs + tt * DP);
+            const f32x4* k4 = reinterpret_cast<const f32x4*>(ks + tt * DP);
+            const f32x4* d4 = reinterpret_cast<const f32x4*>(ds + tt * DP);
+            float g = 1.f;
+            if constexpr (CHD) {
+#pragma unroll
+                for (int r = 0; r < DP; r += 4) {
+                    const f32x4 dv = d4[r >> 2];
+                    st_[r] *= dv[0]; st_[r + 1] *= dv[1]; st_[r + 2] *= dv[2]; st_[r + 3] *= dv[3];
+                }
+            } else {
+                g = gs[tt];
+            }
+            float u = vs[tt * 64 * NW + wv * 64 + lane];
+            if constexpr (DELTA) {
+                float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+#pragma unroll
+                for (int r = 0; r < DP; r += 4) {
+                    const f32x4 kv = k4[r >> 2];
+                    p0 += st_[r] * kv[0]; p1 += st_[r + 1] * kv[1]; p2 += st_[r + 2] * kv[2]; p3 += st_[r + 3] * kv[3];
+                }
+                u = bs[tt] * (u - g * ((p0 + p1) + (p2 + p3)));
+            }
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+            for (int r = 0; r < DP; r += 4) {
+                const f32x4 kv = k4[r >> 2], qv = q4[r >> 2];
+                st_[r] = g * st_[r] + kv[0] * u;
+                st_[r + 1] = g * st_[r + 1] + kv[1] * u;
+                st_[r + 2] = g * st_[r + 2] + kv[2] * u;
+                st_[r + 3] = g * st_[r + 3] + kv[3] * u;
+                a0 += st_[r] * qv[0]; a1 += st_[r + 1] * qv[1]; a2 += st_[r + 2] * qv[2]; a3 += st_[r + 3] * qv[3];
+            }
+            if (live) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = (a0 + a1) + (a2 + a3);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < DP; ++r)
+            if (r < D) Sp[(int64_t)r * Dv] = st_[r];
+    }
+}
+
+}  // namespace hy
+
+void launch_hy_short_conv(const void* x, int ldx, const float* w, const int32_t* tok_seq, const int32_t* q_start,
+                          const int32_t* pos0, const int32_t* slots, void* hist, void* y, int T, int B, int C, int K,
+                          bool silu, bool f32, hipStream_t s) {
+    if (T == 0 || C == 0) return;
+    const dim3 hg(B, (C + 255) / 256);
+    if (f32) {
+        hy::short_conv_kernel<float><<<T, 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu);
+        if (K > 1) hy::conv_hist_kernel<float><<<hg, 256, 0, s>>>((const float*)x, ldx, q_start, pos0, slots, (float*)hist, C, K);
+    } else {
+        hy::short_conv_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu);
+        if (K > 1) hy::conv_hist_kernel<uint16_t><<<hg, 256, 0, s>>>((const uint16_t*)x, ldx, q_start, pos0, slots, (uint16_t*)hist, C, K);
+    }
+}
+
+void launch_hy_delta_prep(const void* y, int ldy, const float* ab, const float* a_log, float* qscale, float* kscale,
+                          float* decay, float* beta, int T, int HK, int H, int D, float q_mul, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    if (f32) hy::delta_prep_kernel<float><<<T, 256, 0, s>>>((const float*)y, ldy, ab, a_log, qscale, kscale, decay, beta, HK, H, D, q_mul);
+    else hy::delta_prep_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)y, ldy, ab, a_log, qscale, kscale, decay, beta, HK, H, D, q_mul);
+}
+
+template <typename T, int DP, bool DELTA, bool CHD>
+static void linear_scan_launch(const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
+                               const float* kscale, float q_mul, const float* decay, const float* beta,
+                               const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
+                               int HK, int H, int D, int Dv, hipStream_t s) {
+    const int NW = Dv > 192 ? 4 : Dv > 128 ? 3 : Dv > 64 ? 2 : 1;
+    const int bytes = (hy::kScanTC * DP * (CHD ? 3 : 2) + hy::kScanTC * 64 * NW + 2 * hy::kScanTC) * 4;
+    auto kern = hy::linear_scan_kernel<T, DP, DELTA, CHD>;
+    if (bytes > 48 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    const dim3 grid(B, H, (Dv + 64 * NW - 1) / (64 * NW));
+    kern<<<grid, 64 * NW, bytes, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0,
+                                      slots, S, o, HK, H, D, Dv);
+}
+
+template <typename T, bool DELTA, bool CHD>
+static bool linear_scan_d(const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
+                          const float* kscale, float q_mul, const float* decay, const float* beta, const int32_t* q_start,
+                          const int32_t* pos0, const int32_t* slots, float* S, float* o, int B, int HK, int H, int D,
+                          int Dv, hipStream_t s) {
+#define HY_LS(DP)                                                                                                     \
+    linear_scan_launch<T, DP, DELTA, CHD>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, \
+                                          pos0, slots, S, o, B, HK, H, D, Dv, s)
+    if (D <= 32) HY_LS(32);
+    else if (D <= 64) HY_LS(64);
+    else if (D <= 128) HY_LS(128);
+    else if (D <= 256) HY_LS(256);
+    else return false;
+#undef HY_LS
+    return true;
+}
+
+// delta: beta != nullptr.  chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
+// Returns false when D has no instantiation (D > 256).
+bool launch_hy_linear_scan(const void* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
+                           const float* kscale, float q_mul, const float* decay, bool chd, const float* beta,
+                           const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
+                           int HK, int H, int D, int Dv, bool f32, hipStream_t s) {
+    if (B == 0) return true;
+    const bool delta = beta != nullptr;
+#define HY_LSD(T, DELTA, CHD)                                                                                        \
+    return linear_scan_d<T, DELTA, CHD>((const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, \
+                                        q_start, pos0, slots, S, o, B, HK, H, D, Dv, s)
+    if (f32) {
+        if (delta && chd) HY_LSD(float, true, true);
+        if (delta) HY_LSD(float, true, false);
+        if (chd) HY_LSD(float, false, true);
+        HY_LSD(float, false, false);
+    } else {
+        if (delta && chd) HY_LSD(uint16_t, true, true);
+        if (delta) HY_LSD(uint16_t, true, false);
+        if (chd) HY_LSD(uint16_t, false, true);
+        HY_LSD(uint16_t, false, false);
+    }
+#undef HY_LSD
+}
+
+}  // namespace chronos

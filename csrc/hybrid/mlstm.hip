@@ -355,7 +355,7 @@ __global__ void __launch_bounds__(256) mlstm_state_scan_vec_kernel(
 template <typename T>
 __global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict__ o, const T* __restrict__ proj, int ldp,
                                                         int g_off, const float* __restrict__ w, T* __restrict__ y,
-                                                        int rows, int H, int Dv, float eps) {
+                                                        int rows, int H, int Dv, float eps, int silu) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (r >= rows) return;
@@ -366,8 +366,10 @@ __global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict_
     for (int i = lane; i < Dv; i += 64) ss += orow[i] * orow[i];
     const float inv = 1.f / sqrtf(wave_sum(ss) / (float)Dv + eps);
     const T* g = proj + t * ldp + g_off + hd * Dv;
-    for (int i = lane; i < Dv; i += 64)
-        st<T>(y + r * Dv + i, orow[i] * inv * w[hd * Dv + i] * sigmoidf_(ld<T>(g + i)));
+    for (int i = lane; i < Dv; i += 64) {
+        const float gv = ld<T>(g + i);
+        st<T>(y + r * Dv + i, orow[i] * inv * w[hd * Dv + i] * (silu ? gv * sigmoidf_(gv) : sigmoidf_(gv)));
+    }
 }
 
 }  // namespace hy
@@ -409,13 +411,19 @@ void launch_hy_mlstm_scan(const void* proj, int ldp, const float* gate_pre, cons
     else mlstm_scan_t<uint16_t>((const uint16_t*)proj, ldp, gate_pre, q_start, pos0, slots, S, n, m, a, b, den, o, B, H, D, Dv, cap, s);
 }
 
-void launch_hy_mlstm_out(const float* o, const void* proj, int ldp, int g_off, const float* w, void* y, int T, int H,
-                         int Dv, float eps, bool f32, hipStream_t s) {
+// silu_gate: the gate columns pass SiLU instead of the sigmoid (the read-out of the linear-state mixers)
+void launch_hy_head_norm_gate(const float* o, const void* proj, int ldp, int g_off, const float* w, void* y, int T, int H,
+                              int Dv, float eps, bool silu_gate, bool f32, hipStream_t s) {
     const int rows = T * H;
     if (rows == 0) return;
     const int blocks = (rows + 3) / 4;
-    if (f32) hy::mlstm_out_kernel<float><<<blocks, 256, 0, s>>>(o, (const float*)proj, ldp, g_off, w, (float*)y, rows, H, Dv, eps);
-    else hy::mlstm_out_kernel<uint16_t><<<blocks, 256, 0, s>>>(o, (const uint16_t*)proj, ldp, g_off, w, (uint16_t*)y, rows, H, Dv, eps);
+    if (f32) hy::mlstm_out_kernel<float><<<blocks, 256, 0, s>>>(o, (const float*)proj, ldp, g_off, w, (float*)y, rows, H, Dv, eps, silu_gate);
+    else hy::mlstm_out_kernel<uint16_t><<<blocks, 256, 0, s>>>(o, (const uint16_t*)proj, ldp, g_off, w, (uint16_t*)y, rows, H, Dv, eps, silu_gate);
+}
+
+void launch_hy_mlstm_out(const float* o, const void* proj, int ldp, int g_off, const float* w, void* y, int T, int H,
+                         int Dv, float eps, bool f32, hipStream_t s) {
+    launch_hy_head_norm_gate(o, proj, ldp, g_off, w, y, T, H, Dv, eps, false, f32, s);
 }
 
 }  // namespace chronos

@@ -120,6 +120,102 @@ __global__ void __launch_bounds__(256) moe_ffn_token_kernel(const T* __restrict_
     for (int i = threadIdx.x; i < d; i += 256) st<T>(out + t * d + i, os[i]);
 }
 
+// One wave per token: the `top` largest of z [T, N] (ties: the lower index), weighted by the softmax over the chosen
+// logits only.  top <= 64 (lane k keeps the k-th choice).
+__global__ void __launch_bounds__(256) moe_select_topk_kernel(const float* __restrict__ z, int32_t* __restrict__ idx,
+                                                              float* __restrict__ wt, int rows, int N, int top) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= rows) return;
+    float c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        c[j] = e < N ? z[t * N + e] : -INFINITY;
+    }
+    float first = 0.f, sum = 0.f, mine = 0.f;  // lane k keeps the k-th chosen logit's exponential
+    for (int k = 0; k < top; ++k) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = lane + 64 * j;
+            if (e < N && (c[j] > bv || (c[j] == bv && e < be))) {
+                bv = c[j]; be = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oe = __shfl_xor(be, o, 64);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov; be = oe;
+            }
+        }
+        if (k == 0) first = bv;  // the largest logit: the softmax's reference point
+        const float ex = expf(bv - first);
+        sum += ex;
+        if (k == lane) {
+            mine = ex;
+            idx[t * top + k] = be;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (lane + 64 * j == be) c[j] = -INFINITY;
+    }
+    if (lane < top) wt[t * top + lane] = mine / sum;
+}
+
+// Gated experts: per token sum_k weight_k * W_down,e ( g sigmoid(slope g) (u + shift) ), g = min(W_gate,e h, limit),
+// u = clamp(W_up,e h, +-limit).  w_gu [E, 2F, d]: gate rows then up rows.  LDS: h (d) | gate, up (2F) | out (d).
+template <typename T>
+__global__ void __launch_bounds__(256) moe_glu_token_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
+                                                            const float* __restrict__ wt, const T* __restrict__ w_gu,
+                                                            const T* __restrict__ w_down, T* __restrict__ out, int d,
+                                                            int F, int E, int top, float limit, float slope,
+                                                            float shift) {
+    extern __shared__ float sm[];
+    float* hs = sm;
+    float* zs = hs + d;
+    float* os = zs + 2 * F;
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < d; i += 256) {
+        hs[i] = ld<T>(h + t * d + i);
+        os[i] = 0.f;
+    }
+    __syncthreads();
+    for (int k = 0; k < top; ++k) {
+        const int e = idx[t * top + k];
+        const float g = wt[t * top + k];
+        if (e < 0 || e >= E) continue;  // (uniform over the workgroup)
+        const T* wu = w_gu + (int64_t)e * 2 * F * d;
+        for (int f = wv; f < 2 * F; f += 4) {
+            const T* wr = wu + (int64_t)f * d;
+            float acc = 0.f;
+            for (int i = lane; i < d; i += 64) acc += ld<T>(wr + i) * hs[i];
+            acc = wave_sum(acc);
+            if (lane == 0) zs[f] = rnd<T>(acc);
+        }
+        __syncthreads();
+        for (int f = threadIdx.x; f < F; f += 256) {
+            const float a = fminf(zs[f], limit), u = fminf(fmaxf(zs[F + f], -limit), limit);
+            zs[f] = rnd<T>(a * sigmoidf_(slope * a) * (u + shift));
+        }
+        __syncthreads();
+        const T* wd = w_down + (int64_t)e * d * F;
+        for (int r = wv; r < d; r += 4) {
+            const T* wr = wd + (int64_t)r * F;
+            float acc = 0.f;
+            for (int i = lane; i < F; i += 64) acc += ld<T>(wr + i) * zs[i];
+            acc = wave_sum(acc);
+            if (lane == 0) os[r] += g * rnd<T>(acc);
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < d; i += 256) st<T>(out + t * d + i, os[i]);
+}
+
 }  // namespace hy
 
 void launch_hy_rowdot(const void*, const void*, const float*, float*, int, int, int, bool, hipStream_t);
@@ -144,6 +240,30 @@ void launch_hy_moe_ffn_token(const void* h, const int32_t* idx, const float* wt,
         auto kern = hy::moe_ffn_token_kernel<uint16_t>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         kern<<<T, 256, bytes, s>>>((const uint16_t*)h, idx, wt, (const uint16_t*)w_up, (const uint16_t*)w_down, (uint16_t*)out, d, F, E, top, act);
+    }
+}
+
+// z: float [T, N] scratch for the router logits (bias added by the projection), N <= 256
+void launch_hy_moe_route_topk(const void* h, const void* w, const float* bias, float* z, int32_t* idx, float* wt, int T,
+                              int d, int N, int top, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    launch_hy_rowdot(h, w, bias, z, T, d, N, f32, s);
+    hy::moe_select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(z, idx, wt, T, N, top);
+}
+
+void launch_hy_moe_glu_token(const void* h, const int32_t* idx, const float* wt, const void* w_gu, const void* w_down,
+                             void* out, int T, int d, int F, int E, int top, float limit, float slope, float shift,
+                             bool f32, hipStream_t s) {
+    if (T == 0) return;
+    const int bytes = (2 * d + 2 * F) * 4;
+    if (f32) {
+        auto kern = hy::moe_glu_token_kernel<float>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<T, 256, bytes, s>>>((const float*)h, idx, wt, (const float*)w_gu, (const float*)w_down, (float*)out, d, F, E, top, limit, slope, shift);
+    } else {
+        auto kern = hy::moe_glu_token_kernel<uint16_t>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<T, 256, bytes, s>>>((const uint16_t*)h, idx, wt, (const uint16_t*)w_gu, (const uint16_t*)w_down, (uint16_t*)out, d, F, E, top, limit, slope, shift);
     }
 }
 

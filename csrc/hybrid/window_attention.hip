@@ -1,0 +1,262 @@
+// window_attention.hip — grouped-query softmax attention over paged keys and values through a sliding window that
+// also keeps each sequence's first tokens, with a learned sink per head in the softmax denominator.
+//
+//   window_prep       per token: per-head RMS norm (float) and rotation (cos / sin from a float table made in double
+//                     precision) of the query heads (in place) and key heads; the values optionally mixed with the
+//                     same token's values of an earlier layer, (1 - lam) v + lam v_first; keys and values written to
+//                     the token's page and slot of kc [NB, BS, G, D] / vc [NB, BS, G, Dv].
+//   window_attention  the general kernel (vector ALUs, float or bfloat16, any sizes): a workgroup takes one sequence,
+//                     one key/value head and up to 16 consecutive query tokens with all the query heads of that
+//                     group (at most 64 (token, head) rows); 64-key tiles of the cache are staged in LDS; lanes are keys for the scores (float
+//                     accumulation, online softmax in float) and value columns for the output.  The key range of a
+//                     tile of queries is [0, keep_first) and [first query - window + 1, last query]; tiles of keys
+//                     between the two are never touched, and each row masks by its own position:
+//                         visible(i, j) = j <= i and (window == 0 or i - j < window or j < keep_first).
+//                     After the last key the sink joins the denominator: l += exp(sink_h - m) (no value), and the
+//                     row is multiplied by sigmoid(gate) when a gate is given.
+// Prompt portions, decode rows and mixed steps are one code path (a decode row is a tile of one token).
+#include <algorithm>
+
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+// LDS: one float row of D per wave.
+template <typename T>
+__global__ void __launch_bounds__(256) window_prep_kernel(
+        T* __restrict__ qkv, int ldq, int H, int G, int D, int Dv, const T* __restrict__ v_first,
+        const float* __restrict__ lam, const int32_t* __restrict__ pos, const int32_t* __restrict__ tok_seq,
+        const int32_t* __restrict__ block_table, int max_blocks, const float* __restrict__ q_norm,
+        const float* __restrict__ k_norm, float eps, const float* __restrict__ cos_sin, int dims, T* __restrict__ kc,
+        T* __restrict__ vc, int BS, T* __restrict__ v_out) {
+    extern __shared__ float wp_smem[];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float* row = wp_smem + wv * D;
+    const int p = pos[t];
+    const int64_t slot = (int64_t)block_table[(int64_t)tok_seq[t] * max_blocks + p / BS] * BS + p % BS;
+    const int half = dims / 2;
+    const float* cs = cos_sin != nullptr ? cos_sin + (int64_t)p * dims : nullptr;
+    T* base = qkv + t * ldq;
+    for (int j = wv; j < H + G; j += 4) {  // heads 0..H-1: queries (in place); H..H+G-1: keys (to the cache)
+        const T* src = base + (int64_t)j * D;
+        const float* nw = j < H ? q_norm : k_norm;
+        float ss = 0.f;
+        for (int i = lane; i < D; i += 64) {
+            const float v = ld<T>(src + i);
+            row[i] = v;
+            ss += v * v;
+        }
+        const float inv = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+        T* dst = j < H ? base + (int64_t)j * D : kc + (slot * G + (j - H)) * D;
+        // (wave-private LDS row: the wave's own writes above are visible to its reads below without a barrier,
+        // the compiler orders LDS accesses of one wave)
+        for (int i = lane; i < D; i += 64) {
+            float v = row[i] * inv * nw[i];
+            if (i < half) v = v * cs[i] - row[i + half] * inv * nw[i + half] * cs[half + i];
+            else if (i < dims) v = v * cs[i - half] + row[i - half] * inv * nw[i - half] * cs[i];
+            st<T>(dst + i, v);
+        }
+    }
+    const float l = v_first != nullptr ? lam[0] : 0.f;
+    const T* vsrc = base + (int64_t)(H + G) * D;
+    for (int i = threadIdx.x; i < G * Dv; i += 256) {
+        float v = ld<T>(vsrc + i);
+        if (v_out != nullptr) st<T>(v_out + t * G * Dv + i, v);
+        if (v_first != nullptr) v = (1.f - l) * v + l * ld<T>(v_first + t * G * Dv + i);
+        st<T>(vc + slot * G * Dv + i, v);
+    }
+}
+
+constexpr int kWaQT = 16;   // query tokens per workgroup at most (fewer when the group has more than 4 heads)
+constexpr int kWaRows = 64; // (token, head) rows per workgroup at most
+constexpr int kWaKT = 64;   // keys per tile
+constexpr int kWaRB = 4;    // rows a wave carries through a tile together
+
+template <typename T> struct WaPad { static constexpr int V = 2; };
+template <> struct WaPad<float> { static constexpr int V = 1; };
+
+// rows = query tokens x R heads of the group.  LDS: K tile [64][D + pad] T | V tile [64][Dv + pad] T |
+// q rows [QT R][D] float | per wave: weights [RB][64] float.
+template <typename T>
+__global__ void __launch_bounds__(256) window_attention_kernel(
+        const T* __restrict__ qkv, int ldq, const T* __restrict__ kc, const T* __restrict__ vc,
+        const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
+        const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
+        T* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int QT) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char wa_smem[];
+    constexpr int PAD = WaPad<T>::V;
+    const int R = H / G;
+    const int b = blockIdx.x, g = blockIdx.z;
+    const int t0 = q_start[b] + blockIdx.y * QT;
+    const int t1 = min(q_start[b + 1], t0 + QT);
+    if (t1 <= t0) return;
+    const int nq = t1 - t0, rows = nq * R;
+    const int ldk = D + PAD, ldv = Dv + PAD;
+    T* Ks = reinterpret_cast<T*>(wa_smem);
+    T* Vs = Ks + kWaKT * ldk;
+    float* Qs = reinterpret_cast<float*>(wa_smem + (((size_t)kWaKT * (ldk + ldv) * sizeof(T) + 15) & ~(size_t)15));
+    float* Ps = Qs + (size_t)kWaRows * D;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float* Pw = Ps + wv * kWaRB * kWaKT;
+    for (int i = threadIdx.x; i < rows * D; i += 256) {
+        const int r = i / D, d = i % D;
+        Qs[i] = ld<T>(qkv + (int64_t)(t0 + r / R) * ldq + (g * R + r % R) * D + d);
+    }
+    const int p_lo = pos[t0], p_hi = pos[t1 - 1];
+    // tokens of a range sit at consecutive positions, so the tile's queries are p_lo .. p_hi
+    const int w_lo = window > 0 ? max(0, p_lo - window + 1) : 0;
+    const int w_start = w_lo / kWaKT * kWaKT;
+    // kept first tokens below the window's first tile: keys [0, k_end) (those from w_start on pass the window tiles'
+    // own test), so no key is ever counted twice
+    const int k_end = window > 0 ? min(keep, w_start) : 0;
+    const int n_keep_tiles = (k_end + kWaKT - 1) / kWaKT;
+    const int n_win_tiles = (p_hi - w_start) / kWaKT + 1;
+    const int NC = (Dv + 63) / 64;
+    // every wave carries its row groups through all tiles: group q of wave wv = rows (q * 4 + wv) * RB ..
+    const int ngroups = (rows + kWaRB - 1) / kWaRB;
+    const int my_groups = (ngroups - wv + 3) / 4;
+    constexpr int MAXG = kWaRows / kWaRB / 4;
+    float m_[MAXG][kWaRB], l_[MAXG][kWaRB], o_[MAXG][kWaRB][4];
+#pragma unroll
+    for (int q = 0; q < MAXG; ++q)
+#pragma unroll
+        for (int r = 0; r < kWaRB; ++r) {
+            m_[q][r] = -INFINITY;
+            l_[q][r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o_[q][r][c] = 0.f;
+        }
+    for (int ti = 0; ti < n_keep_tiles + n_win_tiles; ++ti) {
+        const int j0 = ti < n_keep_tiles ? ti * kWaKT : w_start + (ti - n_keep_tiles) * kWaKT;
+        const int j_end = ti < n_keep_tiles ? min(k_end, j0 + kWaKT) : min(p_hi + 1, j0 + kWaKT);  // keys [j0, j_end)
+        __syncthreads();
+        for (int i = threadIdx.x; i < kWaKT * D; i += 256) {
+            const int kk = i / D, d = i % D, j = j0 + kk;
+            T v;
+            st<T>(&v, 0.f);
+            if (j < j_end) v = kc[(((int64_t)block_table[(int64_t)b * max_blocks + j / BS] * BS + j % BS) * G + g) * D + d];
+            Ks[kk * ldk + d] = v;
+        }
+        for (int i = threadIdx.x; i < kWaKT * Dv; i += 256) {
+            const int kk = i / Dv, d = i % Dv, j = j0 + kk;
+            T v;
+            st<T>(&v, 0.f);
+            if (j < j_end) v = vc[(((int64_t)block_table[(int64_t)b * max_blocks + j / BS] * BS + j % BS) * G + g) * Dv + d];
+            Vs[kk * ldv + d] = v;
+        }
+        __syncthreads();
+        const int j = j0 + lane;
+#pragma unroll
+        for (int q = 0; q < MAXG; ++q) {
+            if (q >= my_groups) break;
+            const int r0 = (q * 4 + wv) * kWaRB;
+            float s[kWaRB] = {0.f, 0.f, 0.f, 0.f};
+            const T* krow = Ks + lane * ldk;
+            for (int d = 0; d < D; ++d) {
+                const float kv = ld<T>(krow + d);
+#pragma unroll
+                for (int r = 0; r < kWaRB; ++r) s[r] += Qs[min(r0 + r, rows - 1) * D + d] * kv;
+            }
+#pragma unroll
+            for (int r = 0; r < kWaRB; ++r) {
+                const int rr = min(r0 + r, rows - 1);
+                const int pi = p_lo + rr / R;
+                const bool vis = j < j_end && j <= pi && (window <= 0 || pi - j < window || j < keep);
+                const float sv = vis ? s[r] * scale : -INFINITY;
+                const float mn = fmaxf(m_[q][r], wave_max(sv));
+                const float pw = mn == -INFINITY ? 0.f : expf(sv - mn);
+                const float corr = m_[q][r] == -INFINITY ? 0.f : expf(m_[q][r] - mn);
+                l_[q][r] = l_[q][r] * corr + wave_sum(pw);
+                m_[q][r] = mn;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) o_[q][r][c] *= corr;
+                Pw[r * kWaKT + lane] = pw;
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int col = c * 64 + lane;
+                if (c < NC && col < Dv) {
+                    float a[kWaRB] = {0.f, 0.f, 0.f, 0.f};
+                    for (int kk = 0; kk < kWaKT; ++kk) {
+                        const float vv = ld<T>(Vs + kk * ldv + col);
+#pragma unroll
+                        for (int r = 0; r < kWaRB; ++r) a[r] += Pw[r * kWaKT + kk] * vv;
+                    }
+#pragma unroll
+                    for (int r = 0; r < kWaRB; ++r) o_[q][r][c] += a[r];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < MAXG; ++q) {
+        if (q >= my_groups) break;
+        const int r0 = (q * 4 + wv) * kWaRB;
+#pragma unroll
+        for (int r = 0; r < kWaRB; ++r) {
+            const int rr = r0 + r;
+            if (rr >= rows) continue;
+            const int64_t t = t0 + rr / R;
+            const int hd = g * R + rr % R;
+            float m = m_[q][r], l = l_[q][r];
+            if (sink != nullptr) {
+                const float sk = sink[hd];
+                const float mn = fmaxf(m, sk);
+                const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+                l = l * corr + expf(sk - mn);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) o_[q][r][c] *= corr;
+            }
+            float f = l > 0.f ? 1.f / l : 0.f;
+            if (gate != nullptr) f *= sigmoidf_(gate[t * H + hd]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int col = c * 64 + lane;
+                if (c < NC && col < Dv) st<T>(out + (t * H + hd) * Dv + col, o_[q][r][c] * f);
+            }
+        }
+    }
+}
+
+}  // namespace hy
+
+void launch_hy_window_prep(void* qkv, int ld, int H, int G, int D, int Dv, const void* v_first, const float* lam,
+                           const int32_t* pos, const int32_t* tok_seq, const int32_t* block_table, int max_blocks,
+                           const float* q_norm, const float* k_norm, float eps, const float* cos_sin, int dims, void* kc,
+                           void* vc, int BS, void* v_out, int T, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    const int bytes = 4 * D * 4;
+    if (f32) hy::window_prep_kernel<float><<<T, 256, bytes, s>>>((float*)qkv, ld, H, G, D, Dv, (const float*)v_first, lam, pos, tok_seq, block_table, max_blocks, q_norm, k_norm, eps, cos_sin, dims, (float*)kc, (float*)vc, BS, (float*)v_out);
+    else hy::window_prep_kernel<uint16_t><<<T, 256, bytes, s>>>((uint16_t*)qkv, ld, H, G, D, Dv, (const uint16_t*)v_first, lam, pos, tok_seq, block_table, max_blocks, q_norm, k_norm, eps, cos_sin, dims, (uint16_t*)kc, (uint16_t*)vc, BS, (uint16_t*)v_out);
+}
+
+// LDS bytes of the general kernel; the caller checks it against the 160 KB of a CU.
+size_t hy_window_attention_lds(int D, int Dv, bool f32) {
+    const size_t e = f32 ? 4 : 2, pad = f32 ? 1 : 2;
+    const size_t tiles = ((size_t)hy::kWaKT * (D + pad + Dv + pad) * e + 15) & ~(size_t)15;
+    return tiles + ((size_t)hy::kWaRows * D + 4 * hy::kWaRB * hy::kWaKT) * 4;
+}
+
+void launch_hy_window_attention(const void* qkv, int ld, const void* kc, const void* vc, const int32_t* block_table,
+                                int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
+                                const float* gate, void* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
+                                float scale, int window, int keep, bool f32, hipStream_t s) {
+    if (B == 0 || max_q == 0) return;
+    const int bytes = (int)hy_window_attention_lds(D, Dv, f32);
+    const int R = H / G;   // the caller has checked R <= 64, Dv <= 256 and the LDS size
+    const int QT = std::max(1, std::min(hy::kWaQT, hy::kWaRows / R));
+    const dim3 grid(B, (max_q + QT - 1) / QT, G);
+    if (f32) {
+        auto kern = hy::window_attention_kernel<float>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<grid, 256, bytes, s>>>((const float*)qkv, ld, (const float*)kc, (const float*)vc, block_table, max_blocks, q_start, pos, sink, gate, (float*)out, H, G, D, Dv, BS, scale, window, keep, QT);
+    } else {
+        auto kern = hy::window_attention_kernel<uint16_t>;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        kern<<<grid, 256, bytes, s>>>((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc, block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, H, G, D, Dv, BS, scale, window, keep, QT);
+    }
+}
+
+}  // namespace chronos

@@ -461,7 +461,7 @@ def mix_delta_rule(model, li: int, spec: DeltaRuleSpec, w: dict, h, meta: StepMe
     C = 2 * HK * D + H * Dv
     proj = hops.matmul(h, w["w_proj"])          # q | k | v | g
     ab = hops.rowdot(h, w["w_ab"], w["b_ab"])   # decay and write-strength pre-activations, float32
-    y = hops.short_conv(proj, w["taps"], meta.q_start, meta.pos0, meta.slots, cache.hist[li], True)
+    y = hops.short_conv(proj, w["taps"], meta.tok_seq, meta.q_start, meta.pos0, meta.slots, cache.hist[li], True)
     qscale, kscale, decay, beta = hops.delta_prep(y, ab, w["a_log"], HK, H, D, D ** -0.5)
     o = hops.linear_scan(y, 0, HK * D, 2 * HK * D, qscale, kscale, 1.0, decay, beta, meta.q_start, meta.pos0,
                          meta.slots, cache.S[li], HK, H, D, Dv)

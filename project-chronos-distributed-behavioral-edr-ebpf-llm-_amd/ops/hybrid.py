@@ -175,9 +175,9 @@ def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale: 
                                 act_dtype)
 
 
-def short_conv(x, w, q_start, pos0, slots, hist, silu: bool = True):
+def short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu: bool = True):
     if _gpu(x):
-        return _k().hy_short_conv(x, w, q_start, pos0, slots, hist, silu)
+        return _k().hy_short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu)
     return ref.short_conv(x, w, q_start, pos0, slots, hist, silu)
 
 
