@@ -1,0 +1,473 @@
+"""Kalesun through the framework (registry -> engine -> block manager / state slots -> step batches -> ops) against
+the plain token-by-token oracle of tests/oracles/kalesun_plain.py.
+
+CPU runs take the ops' PyTorch path, the ``cuda`` parametrisations (marked gpu) the HIP kernels; both go through the
+same engine code.  Sizes are deliberately unlike each other: head groups of 1, 2 and 3, key/value heads equal to the
+query heads, windows shorter than a page and longer than two, no kept tokens, rotation of all and of a few columns,
+convolutions of 1 to 5 taps, routers that take one expert or all of them, a residual weight that is not 2.
+"""
+import copy
+import json
+
+import pytest
+import torch
+
+from tests.oracles import kalesun_plain as plain
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+TOL = {"fp32": 2e-4, "bf16": 0.1}
+
+
+def _attn(heads=4, kv_heads=2, dim=12, vdim=20, scale=0.4, size=21, keep=3, dims=8, base=3000.0, scaling=True,
+          v_mix=True):
+    mx = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, v_mix=v_mix)
+    if size:
+        mx["mask"] = dict(size=size, keep_first=keep)
+    if dims:
+        mx["rot"] = dict(base=base, dims=dims)
+        if scaling:
+            mx["rot"]["scaling"] = dict(factor=4.0, low=1.0, high=4.0, original=40)
+    return dict(type="attention", mixer=mx)
+
+
+def _delta(heads=4, kv_heads=2, dim=8, vdim=12, conv=3):
+    return dict(type="delta", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, conv=conv))
+
+
+def _gla(heads=3, dim=8, vdim=20, tau=8.0, rank=5):
+    return dict(type="gla", mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=tau, rank=rank))
+
+
+def _dense(ff=40, limit=1.2):
+    return dict(kind="dense", ff=ff, limit=limit)
+
+
+def _moe(experts=5, top=2, ff=24, limit=0.9):
+    return dict(kind="moe", expert=dict(ff=ff, limit=limit), router=dict(experts=experts, top=top))
+
+
+def _config(layers, width=64, vocab=97, alpha=1.6, eps=1e-5):
+    return dict(architecture="Kalesun", vocab=vocab, width=width, postln_alpha=alpha, norm=dict(eps=eps),
+                layers=[dict(l[0], mlp=l[1]) for l in layers])
+
+
+MIXED = _config([(_delta(), _moe()), (_attn(), _dense()), (_gla(), None),
+                 (_attn(heads=4, kv_heads=2, dim=16, vdim=20, size=40, keep=0, dims=16, scaling=False, scale=0.2), _moe(3, 3, 16)),
+                 (_delta(heads=2, kv_heads=2, dim=20, vdim=6, conv=5), _dense(24, 3.0)),
+                 (_attn(heads=2, kv_heads=1, dim=12, vdim=20, size=7, keep=9, dims=4, v_mix=False), _moe(4, 1, 8))])
+
+
+def _model(cfg_dict, device, dtype="fp32", seed=0, tensors=None):
+    from chronos.models import kalesun
+    from chronos.models.hybrid import HybridDecoder
+
+    cfg = kalesun.config_from_dict(cfg_dict, max_position=1024)
+    if tensors is None:
+        tensors = kalesun.random_tensors(cfg, seed)
+        if dtype == "bf16":  # routers far from close calls: a choice flipped by rounding moves every later position
+            for k in tensors:
+                if k.endswith("mlp.router"):
+                    tensors[k] = tensors[k] * 8
+    at = torch.float32 if dtype == "fp32" else torch.bfloat16
+    return HybridDecoder(cfg, kalesun.pack_weights(cfg, tensors, device, at), device, 1024, at), tensors
+
+
+def _engine(cfg_dict, device, dtype="fp32", slots=4, max_len=512, blocks=0, seed=0, tensors=None, **kw):
+    from chronos.brain.engine.engine import Engine, EngineConfig
+
+    model, tensors = _model(cfg_dict, device, dtype, seed, tensors)
+    bs = kw.pop("block_size", 16)
+    ec = EngineConfig(model="kalesun-test", device=device, dtype=dtype, max_slots=slots, block_size=bs,
+                      max_model_len=max_len, kv_blocks=blocks or slots * (max_len // bs) + 1, warm_formats=(), **kw)
+    return Engine(ec, model=model), tensors
+
+
+def _errs(got, want):
+    """Per position: the spread of the difference over the vocabulary relative to the spread of the logits."""
+    d = got.double() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def _err(got, want):
+    return float(_errs(got, want).max())
+
+
+def _bad(got, want, dtype):
+    """float32: the worst position against the tolerance.  bfloat16: rounding can flip a close router choice at a
+    single position of these tiny random models, so the 85th percentile of the positions is held to the tolerance
+    (a fault of a mechanism, a cache or a schedule moves far more positions than that)."""
+    e = _errs(got, want)
+    if dtype == "fp32" or e.numel() < 8:
+        return float(e.max()) >= TOL[dtype] * (1 if dtype == "fp32" else 4)
+    return float(e.sort().values[int(0.85 * (e.numel() - 1))]) >= TOL[dtype]
+
+
+def _tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def _replay(eng, schedule, reqs):
+    """schedule: list of steps, each [(request name, count)].  Returns {name: logits of every token}."""
+    from chronos.brain.engine.replay import TraceSession
+
+    ses = TraceSession(eng)
+    at = {k: 0 for k in reqs}
+    out = {k: [] for k in reqs}
+    for step in schedule:
+        entries, end = [], []
+        for name, count in step:
+            lo = at[name]
+            entries.append(dict(id=name, tokens=reqs[name][lo:lo + count], want=list(range(count))))
+            at[name] = lo + count
+            if at[name] == len(reqs[name]):
+                end.append(name)
+        logits = ses.step(entries, end)
+        k = 0
+        for name, count in step:
+            out[name].append(logits[k:k + count])
+            k += count
+    assert not ses.live
+    return {k: torch.cat(v) for k, v in out.items()}
+
+
+def _want(cfg, tensors, toks):
+    return plain.run(cfg, tensors, toks)[0]
+
+
+# ---- each mechanism alone, layer by layer -------------------------------------------------------------------------
+SINGLE = [(_attn(), None), (_attn(heads=3, kv_heads=3, dim=6, vdim=4, size=0, dims=6, scaling=False, v_mix=False), None),
+          (_attn(heads=6, kv_heads=1, dim=10, vdim=70, size=5, keep=0, dims=0), _dense()),
+          (_attn(heads=2, kv_heads=2, dim=4, vdim=2, size=1, keep=2, dims=2, scale=2.0), None),
+          (_delta(), None), (_delta(heads=1, kv_heads=1, dim=5, vdim=3, conv=1), None),
+          (_delta(heads=6, kv_heads=2, dim=20, vdim=70, conv=2), _moe()), (_gla(), None),
+          (_gla(heads=1, dim=33, vdim=5, tau=1.0, rank=1), _dense(8, 0.3)), (_gla(), _moe(2, 2, 8)),
+          (_delta(), _moe(1, 1, 16, 5.0))]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("layer", SINGLE)
+def test_single_layer_and_residual_stream(device, layer):
+    cfg = _config([layer, layer])
+    model, tensors = _model(cfg, device)
+    toks = _tokens(37, cfg["vocab"], 3)
+    taps = []
+    model.layer_tap = lambda li, x: taps.append(x.detach().clone().cpu())
+    cache = model.make_cache(8, 16, 2)
+    sb = model.prefill_batch([toks], [0], [[1, 2, 3]], [1], want=list(range(len(toks))))
+    got = model.forward(sb, cache).cpu()
+    want, per_layer = plain.run(cfg, tensors, toks)
+    for li, x in enumerate(taps):
+        assert float((x.double() - per_layer[li]).abs().max()) < 2e-4 * float(per_layer[li].abs().max()), f"layer {li}"
+    assert _err(got, want) < TOL["fp32"]
+
+
+def test_rotation_frequencies_follow_the_wavelength_rule():
+    from chronos.models.hybrid import rope_cos_sin
+
+    rot = dict(base=500.0, dims=16, scaling=dict(factor=6.0, low=1.0, high=3.0, original=50))
+    table = rope_cos_sin(500.0, 16, 64, "cpu", (6.0, 1.0, 3.0, 50.0)).double()
+    for i in range(8):
+        f = plain.rope_frequency(i, 16, 500.0, rot["scaling"])
+        p = torch.arange(64, dtype=torch.float64)
+        assert float((table[:, i] - torch.cos(p * f)).abs().max()) < 1e-6
+        assert float((table[:, 8 + i] - torch.sin(p * f)).abs().max()) < 1e-6
+    kinds = {("same" if abs(plain.rope_frequency(i, 16, 500.0, rot["scaling"]) / 500.0 ** (-2 * i / 16) - 1) < 1e-12
+              else "slow" if abs(plain.rope_frequency(i, 16, 500.0, rot["scaling"]) * 6 / 500.0 ** (-2 * i / 16) - 1) < 1e-12
+              else "between") for i in range(8)}
+    assert kinds == {"same", "slow", "between"}, "the test must cover all three branches"
+
+
+# ---- the visible set of the windowed attention, key by key --------------------------------------------------------
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("window,keep", [(9, 3), (16, 0), (64, 17), (70, 70), (1, 1), (0, 0), (130, 2)])
+def test_window_visible_set(device, window, keep):
+    """Zero queries make every visible key weigh the same, and one-hot values make the output of a query its
+    visibility pattern: out[i, j] = 1 / (visible(i) + exp(sink)) for the keys j that i sees, else 0.  Prompt portions
+    that start and end anywhere beside decode rows, pages dealt out of order."""
+    from chronos.ops import hybrid as hops
+
+    dt = torch.float32
+    ctx, bs, H, G, D = 200, 16, 2, 1, 8
+    nb = ctx // bs + 2
+    kc = torch.randn(nb, bs, G, D, dtype=dt)
+    vc = torch.zeros(nb, bs, G, ctx, dtype=dt)
+    pages = list(range(nb - 1, 0, -1))
+    for j in range(ctx):
+        vc[pages[j // bs], j % bs, 0, j] = 1.0
+    sink = torch.tensor([0.3, -1.0])
+    for lo, hi in [(0, 200), (0, 1), (63, 65), (64, 130), (127, 200), (199, 200), (5, 6), (150, 151)]:
+        n = hi - lo
+        qkv = torch.zeros(n, H * D, dtype=dt)
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)  # noqa: E731
+        bt = torch.zeros(2, nb, dtype=torch.int32)
+        bt[1, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        # (sequence 0 of the batch brings nothing; the portion belongs to sequence 1)
+        out = hops.window_attention(qkv.to(device), kc.to(device), vc.to(device), bt.to(device), i32([0, 0, n]),
+                                    i32(list(range(lo, hi))), sink.to(device), None, 1.0, window, keep, H, dt, n)
+        out = out.view(n, H, ctx).cpu()
+        for r, i in enumerate(range(lo, hi)):
+            vis = torch.tensor([1.0 if plain.visible(i, j, dict(size=window, keep_first=keep) if window else None) else 0.0
+                                for j in range(ctx)])
+            for h in range(H):
+                want = vis / (vis.sum() + torch.exp(sink[h]))
+                assert float((out[r, h] - want).abs().max()) < 1e-6, (lo, hi, i, h)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("decode", [False, True])
+def test_sharp_softmax_around_the_window_edges(device, decode):
+    """A large score scale lets single keys carry the answer: a key that is one position outside the window, a kept
+    first token that is dropped, or a sink that is left out moves the logits.  Window shorter than a page in one
+    layer and longer than two in the other; the sequence runs far past both."""
+    cfg = _config([(_attn(heads=2, kv_heads=1, dim=8, vdim=8, scale=5.0, size=11, keep=2, dims=4), None),
+                   (_attn(heads=2, kv_heads=1, dim=8, vdim=8, scale=3.0, size=37, keep=5, dims=8), _dense(16))], width=32)
+    eng, tensors = _engine(cfg, device, max_len=256)
+    toks = _tokens(230, cfg["vocab"], 2)
+    sched = [[("r0", 8)]] + [[("r0", 1)] for _ in range(222)] if decode else [[("r0", 33)], [("r0", 2)], [("r0", 195)]]
+    got = _replay(eng, sched, {"r0": toks})["r0"]
+    assert _err(got.cpu(), _want(cfg, tensors, toks)) < TOL["fp32"]
+    no_sink = {k: (v - 30 if k.endswith("sink") else v) for k, v in tensors.items()}
+    assert _err(_want(cfg, no_sink, toks[:40]), _want(cfg, tensors, toks[:40])) > 1e-2, "the test must feel the sink"
+
+
+# ---- schedules: whole prompts, decoding, portions, mixed batches ---------------------------------------------------
+def _requests(cfg, lens, seed=0):
+    return {f"r{i}": _tokens(n, cfg["vocab"], seed + i) for i, n in enumerate(lens)}
+
+
+def _check(eng, tensors, cfg, schedule, reqs, dtype):
+    got = _replay(eng, schedule, reqs)
+    for name, toks in reqs.items():
+        want = _want(cfg, tensors, toks)
+        assert not _bad(got[name].cpu(), want, dtype), (name, _errs(got[name].cpu(), want))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_prefill_equals_token_by_token(device, dtype):
+    eng, tensors = _engine(MIXED, device, dtype)
+    reqs = _requests(MIXED, [75, 1, 18])
+    sched = [[("r0", 75)], [("r1", 1)]] + [[("r2", 1)] for _ in range(18)]
+    _check(eng, tensors, MIXED, sched, reqs, dtype)
+    # the same prompt once more, a little of it at once and the rest decoded: the slot and pages are reused, and the
+    # decoded tokens pass every window
+    sched = [[("r0", 13)]] + [[("r0", 1)] for _ in range(62)]
+    _check(eng, tensors, MIXED, sched, {"r0": reqs["r0"]}, dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_portions_of_every_size(device):
+    eng, tensors = _engine(MIXED, device)
+    reqs = _requests(MIXED, [100], seed=5)
+    cuts = [3, 2, 16, 2, 15, 17, 2, 31, 1, 1, 2, 7, 1]
+    assert sum(cuts) == 100
+    _check(eng, tensors, MIXED, [[("r0", c)] for c in cuts], reqs, "fp32")
+    _check(eng, tensors, MIXED, [[("r0", 2)] for _ in range(50)], reqs, "fp32")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_mixed_batches_with_reused_pages_and_slots(device, dtype):
+    """Four slots and a pool of 14 pages (block 0 is scratch) for six requests of 212 tokens in all: requests end,
+    their pages and slots go to new ones (whose state and convolution history must start from zero); portions run
+    beside single decoded tokens."""
+    eng, tensors = _engine(MIXED, device, dtype, slots=4, max_len=128, blocks=15)
+    reqs = _requests(MIXED, [70, 9, 33, 1, 40, 59], seed=11)
+    sched = [[("r0", 3), ("r1", 1)],
+             [("r0", 30), ("r1", 1), ("r2", 2)],
+             [("r0", 1), ("r1", 2), ("r2", 29), ("r3", 1)],
+             [("r0", 1), ("r1", 1), ("r2", 1), ("r4", 17)],
+             [("r0", 16), ("r1", 4), ("r2", 1), ("r4", 1)],      # r1, r2 end
+             [("r0", 1), ("r4", 1), ("r5", 2)],
+             [("r0", 18), ("r4", 21), ("r5", 31)],               # r0, r4 end
+             [("r5", 1)]] + [[("r5", 1)] for _ in range(25)]
+    _check(eng, tensors, MIXED, sched, reqs, dtype)
+    assert eng.blocks.free == 14 and len(eng.free_slots) == 4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batch_members_do_not_see_each_other(device):
+    eng, tensors = _engine(MIXED, device)
+    reqs = _requests(MIXED, [21, 64, 5], seed=21)
+    alone = {k: _replay(eng, [[(k, len(v))]], {k: v})[k] for k, v in reqs.items()}
+    together = _replay(eng, [[("r0", 21), ("r1", 64), ("r2", 5)]], reqs)
+    for k in reqs:
+        assert _err(together[k], alone[k]) < 1e-5
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_a_request_may_sit_out_steps(device):
+    eng, tensors = _engine(MIXED, device)
+    reqs = _requests(MIXED, [30, 26], seed=31)
+    sched = [[("r0", 7)], [("r1", 5)], [("r1", 1)], [("r0", 2), ("r1", 1)], [("r1", 19)], [("r0", 21)]]
+    _check(eng, tensors, MIXED, sched, reqs, "fp32")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_page_borders_and_first_tokens(device):
+    """Every position from just before a page border to just after it, decoded and in portions that start and end at
+    the border; the first tokens of a sequence one by one (zero state, zero-padded convolution, a lone key beside the
+    sink)."""
+    cfg = _config([(_attn(scale=3.0, size=18, keep=1), _dense()), (_delta(conv=4), None), (_gla(), None)], width=48)
+    eng, tensors = _engine(cfg, device, block_size=16)
+    toks = _tokens(52, cfg["vocab"], 8)
+    want = _want(cfg, tensors, toks)
+    for sched in ([[("r0", 1)] for _ in range(52)],
+                  [[("r0", 16)], [("r0", 16)], [("r0", 15)], [("r0", 2)], [("r0", 3)]],
+                  [[("r0", 15)], [("r0", 2)], [("r0", 30)], [("r0", 5)]]):
+        assert _err(_replay(eng, sched, {"r0": toks})["r0"].cpu(), want) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding_carries_the_state(device):
+    """Strong decays on one side and none on the other, write strengths near one: 160 decoded tokens after three
+    portions, against the oracle."""
+    from chronos.models import kalesun
+
+    cfg = _config([(_delta(heads=2, kv_heads=1, dim=8, vdim=8, conv=4), None), (_gla(heads=2, dim=8, vdim=8, tau=2.0), _dense(16))], width=32)
+    t = kalesun.random_tensors(kalesun.config_from_dict(cfg), 4)
+    t["l0.mix.A_log"] = torch.tensor([-6.0, 1.0]).to(torch.bfloat16)
+    t["l0.mix.b"] = t["l0.mix.b"] * 20
+    t["l1.mix.a2.b"] = torch.cat([torch.full((8,), 9.0), torch.full((8,), -3.0)]).to(torch.bfloat16)
+    eng, tensors = _engine(cfg, device, tensors=t)
+    toks = _tokens(210, cfg["vocab"], 6)
+    sched = [[("r0", 7)], [("r0", 2)], [("r0", 41)]] + [[("r0", 1)] for _ in range(160)]
+    assert _err(_replay(eng, sched, {"r0": toks})["r0"].cpu(), _want(cfg, tensors, toks)) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_router_weights_are_the_softmax_over_the_chosen(device):
+    """A bias that lifts the weakest experts above the strongest decides the choice, and the weights sum to one over
+    the chosen experts only."""
+    from chronos.models import kalesun
+    from chronos.ops import hybrid as hops
+
+    cfg = _config([(_gla(), _moe(5, 2, 16))], width=32)
+    t = kalesun.random_tensors(kalesun.config_from_dict(cfg), 9)
+    t["l0.mlp.router.b"] = torch.tensor([0.0, 6.0, 0.0, 0.0, 5.0]).to(torch.bfloat16)
+    eng, tensors = _engine(cfg, device, tensors=t)
+    toks = _tokens(20, cfg["vocab"], 1)
+    assert _err(_replay(eng, [[("r0", 20)]], {"r0": toks})["r0"].cpu(), _want(cfg, tensors, toks)) < TOL["fp32"]
+    t2 = dict(t)
+    t2["l0.mlp.router.b"] = torch.zeros(5).to(torch.bfloat16)
+    assert _err(_want(cfg, t2, toks), _want(cfg, tensors, toks)) > 1e-2, "the test must be sensitive"
+    h = torch.randn(6, 32, device=device)
+    idx, wt = hops.moe_route_topk(h, t["l0.mlp.router"].float().to(device), t["l0.mlp.router.b"].float().to(device), 2)
+    assert sorted(idx[0].tolist()) == [1, 4] and torch.allclose(wt.sum(-1).cpu(), torch.ones(6))
+
+
+# ---- generation through the engine's own entry point and scheduler ------------------------------------------------
+def _greedy(cfg, tensors, prompt, n):
+    m = plain.Plain(cfg, tensors)
+    logits = None
+    for t in prompt:
+        logits = m.step(int(t))
+    out = []
+    for _ in range(n):
+        out.append(int(logits.argmax()))
+        logits = m.step(out[-1])
+    return out
+
+
+GEN = _config([(_delta(heads=2, kv_heads=1, dim=8, vdim=8), _moe(3, 2, 16)), (_attn(heads=2, kv_heads=1, dim=8, vdim=8, size=12, keep=2, dims=4), _dense(32)),
+               (_gla(heads=2, dim=8, vdim=8), None), (_attn(heads=2, kv_heads=1, dim=8, vdim=8, size=20, keep=0, dims=8), None)],
+              width=32, vocab=61)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(device, graphs):
+    """submit() -> admission -> prefill / mixed steps -> decode bursts -> harvest, five requests over two slots and a
+    small page pool (slots and pages are reused, arrivals join running decodes), greedy tokens equal to the oracle's."""
+    if graphs and device == "cpu":
+        pytest.skip("graphs are a GPU feature")
+    from chronos.models import kalesun
+
+    t = kalesun.random_tensors(kalesun.config_from_dict(GEN), 3)
+    t["embed"] = t["embed"] * 3   # logits far enough apart for a stable argmax
+    eng, tensors = _engine(GEN, device, slots=2, max_len=96, blocks=9, tensors=t, use_graphs=graphs, decode_burst=4,
+                           max_prefill_tokens=24, mixed_prefill_tokens=8, prefill_ramp=0)
+    prompts = [_tokens(n, 59, 30 + n) for n in (5, 31, 12, 2, 40)]   # (ids 59 and 60 are the byte tokenizer's specials)
+    reqs = [eng.submit(p, num_predict=9) for p in prompts[:3]]
+    eng.step()
+    eng.step()
+    reqs += [eng.submit(p, num_predict=9) for p in prompts[3:]]
+    eng.run_until_idle(max_steps=2000)
+    for r, p in zip(reqs, prompts):
+        assert r.done_reason in ("length", "stop"), (r.done_reason, r.error)
+        want = _greedy(GEN, tensors, p, 9)
+        n = len(r.out_ids)
+        # (the engine's free-text automaton spends the last token of the budget on the end-of-text token)
+        assert n >= 8 and r.out_ids == want[:n], (r.out_ids, want)
+    assert eng.blocks.free == 8 and len(eng.free_slots) == 2
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_compaction_and_preemption_carry_the_state(device):
+    """Requests that finish at different times leave holes in the low slots, so running sequences are moved down
+    (recurrent state and convolution history move with them); a page pool too small for all of them forces recompute
+    preemption.  Greedy tokens must equal the oracle's throughout."""
+    from chronos.models import kalesun
+
+    t = kalesun.random_tensors(kalesun.config_from_dict(GEN), 5)
+    t["embed"] = t["embed"] * 3
+    prompts = [_tokens(n, 59, 50 + n) for n in (4, 6, 9, 30)]
+    budgets = [3, 5, 24, 26]
+    eng, tensors = _engine(GEN, device, slots=4, max_len=96, tensors=t, use_graphs=False, decode_burst=2, prefill_ramp=0)
+    reqs = [eng.submit(p, num_predict=n) for p, n in zip(prompts, budgets)]
+    eng.run_until_idle(max_steps=2000)
+    assert eng.stats["compactions"] >= 1
+    for r, p, n in zip(reqs, prompts, budgets):
+        want = _greedy(GEN, tensors, p, n)
+        assert len(r.out_ids) >= n - 1 and r.out_ids == want[:len(r.out_ids)], (r.out_ids, want)
+    eng, _ = _engine(GEN, device, slots=4, max_len=96, blocks=6, tensors=tensors, use_graphs=False, decode_burst=2,
+                     prefill_ramp=0, kv_alloc="lazy", kv_lookahead=2, kv_watermark=0.0)
+    reqs = [eng.submit(p, num_predict=n) for p, n in zip(prompts, budgets)]
+    eng.run_until_idle(max_steps=4000)
+    assert eng.stats["preemptions"] >= 1
+    for r, p, n in zip(reqs, prompts, budgets):
+        assert r.done_reason in ("length", "stop"), (r.done_reason, r.error)
+        want = _greedy(GEN, tensors, p, n)
+        assert len(r.out_ids) >= n - 1 and r.out_ids == want[:len(r.out_ids)], (r.out_ids, want)
+
+
+def test_registry_reads_the_checkpoint_layout(tmp_path):
+    from chronos.models import kalesun, registry
+
+    cfg = kalesun.config_from_dict(MIXED)
+    tensors = kalesun.random_tensors(cfg, 1)
+    kalesun.save(cfg, tensors, str(tmp_path))
+    saved = json.load(open(tmp_path / "config.json"))
+    for l in saved["layers"]:   # the decay projection's rank is read from the tensor's shape
+        l["mixer"].pop("rank", None)
+    json.dump(saved, open(tmp_path / "config.json", "w"))
+    assert registry.family_of(str(tmp_path)).name == "kalesun"
+    model = registry.build_model(str(tmp_path), "cpu", dtype="fp32", max_position=64)
+    assert [l.mixer.rank for l in model.cfg.layers if l.mixer.kind == "gla"] == [5]
+    toks = _tokens(9, cfg.vocab_size, 0)
+    sb = model.prefill_batch([toks], [0], [[1]], [0], want=list(range(9)))
+    assert _err(model.forward(sb, model.make_cache(2, 16, 1)), _want(MIXED, tensors, toks)) < TOL["fp32"]
+    bad = copy.deepcopy(MIXED)
+    bad["layers"][0]["type"] = "conv"
+    with pytest.raises(ValueError):
+        kalesun.config_from_dict(bad)
+    assert "kalesun-tiny" in registry.family_of("kalesun-tiny").presets()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("width", [512, 1024])
+def test_wide_model_on_the_routed_projections(width):
+    """Widths at which single decode rows take the framework's GEMV and the projections its tiled GEMMs: bfloat16
+    prefill against token-by-token decoding against the oracle."""
+    cfg = _config([(_delta(heads=4, kv_heads=2, dim=64, vdim=128, conv=4), _moe(4, 2, 128, 7.0)),
+                   (_attn(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.125, size=24, keep=4, dims=32), _dense(1024, 7.0)),
+                   (_gla(heads=4, dim=64, vdim=128, tau=16.0, rank=16), _dense(512, 7.0))], width=width, vocab=320)
+    eng, tensors = _engine(cfg, "cuda", "bf16", max_len=128)
+    toks = _tokens(40, 320, 3)
+    want = _want(cfg, tensors, toks)
+    for sched in ([[("r0", 40)]], [[("r0", 9)]] + [[("r0", 1)] for _ in range(31)]):
+        got = _replay(eng, sched, {"r0": toks})["r0"].cpu()
+        assert not _bad(got, want, "bf16"), _errs(got, want)
