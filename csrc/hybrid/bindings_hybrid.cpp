@@ -44,7 +44,7 @@ void launch_hy_head_norm_gate(const float*, const void*, int, int, const float*,
 void launch_hy_window_prep(void*, int, int, int, int, int, const void*, const float*, const int32_t*, const int32_t*,
                            const int32_t*, int, const float*, const float*, float, const float*, int, void*, void*, int,
                            void*, int, bool, hipStream_t);
-size_t hy_window_attention_lds(int, int, bool);
+int hy_window_rows_cap(int, int, int, bool);
 void launch_hy_window_attention(const void*, int, const void*, const void*, const int32_t*, int, const int32_t*,
                                 const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
                                 int, int, bool, hipStream_t);
@@ -57,8 +57,10 @@ bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const 
                            int, bool, hipStream_t);
 void launch_hy_moe_route_topk(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
                               hipStream_t);
+void launch_hy_moe_glu_grouped(const uint16_t*, const int32_t*, const float*, const uint16_t*, const uint16_t*, uint16_t*,
+                               int32_t*, uint16_t*, uint16_t*, int, int, int, int, int, float, float, float, hipStream_t);
 void launch_hy_moe_glu_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
-                             int, int, float, float, float, bool, hipStream_t);
+                             int, int, float, float, float, bool, bool, hipStream_t);
 }  // namespace chronos
 
 namespace {
@@ -383,7 +385,7 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
     const int64_t T = qkv.size(0), G = kc.size(2), D = kc.size(3), Dv = vc.size(3);
     need(H >= 1 && H % G == 0 && qkv.size(1) >= H * D && vc.size(2) == G && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "window_attention: shapes");
     need(H / G <= 64 && Dv <= 256, "window_attention: at most 64 query heads per key/value head and 256 value columns");
-    need(chronos::hy_window_attention_lds((int)D, (int)Dv, f32(qkv)) <= 160 * 1024, "window_attention: a key tile and 64 query rows must fit the LDS");
+    need(chronos::hy_window_rows_cap((int)(H / G), (int)D, (int)Dv, f32(qkv)) > 0, "window_attention: a key tile and a group's query rows must fit the LDS");
     i32(block_table, "window_attention: block_table"); i32(q_start, "window_attention: q_start"); i32(pos, "window_attention: pos");
     const int64_t B = q_start.numel() - 1;
     need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T && window >= 0 && keep >= 0, "window_attention: metadata");
@@ -480,7 +482,7 @@ std::tuple<Tensor, Tensor> hy_moe_route_topk(const Tensor& h, const Tensor& w, c
 }
 
 Tensor hy_moe_glu_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, const Tensor& w_gu, const Tensor& w_down,
-                      double limit, double slope, double shift) {
+                      double limit, double slope, double shift, bool tiled) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
     same_act(h, w_gu, "moe_glu_ffn: h and experts in one activation dtype");
     same_act(h, w_down, "moe_glu_ffn: h and experts in one activation dtype");
@@ -489,11 +491,27 @@ Tensor hy_moe_glu_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, cons
     need(w_gu.size(1) == 2 * F && w_gu.size(2) == d && w_down.size(0) == E && w_down.size(1) == d, "moe_glu_ffn: expert shapes");
     i32(idx, "moe_glu_ffn: idx"); flt(wt, "moe_glu_ffn: weights");
     need(idx.dim() == 2 && idx.size(0) == T && wt.sizes() == idx.sizes(), "moe_glu_ffn: idx / weights [T, top]");
-    need((2 * d + 2 * F) * 4 <= 160 * 1024, "moe_glu_ffn: a token's rows must fit the LDS");
     auto out = at::empty_like(h);
+    // bfloat16 with tile-sized widths and more than a few tokens: the grouped MFMA GEMMs over the tile-ordered copy
+    // of the gate / up rows; otherwise the token-parallel kernel (which reads either row order)
+    need(!tiled || (!f32(h) && d % 128 == 0 && F % 128 == 0), "moe_glu_ffn: the tile order is for bfloat16 experts with d and F on the 128 grid");
+    if (tiled && E <= 256 && T * idx.size(1) >= 4 * E) {
+        const int top = (int)idx.size(1), items = (int)T * top;
+        const int maxTiles = chronos::hy_moe_max_tiles(items, (int)E);
+        auto meta = at::empty({1 + (int64_t)maxTiles + (int64_t)maxTiles * 128 + items}, h.options().dtype(at::kInt));
+        auto z = at::empty({(int64_t)maxTiles * 128, F}, h.options());
+        auto yrows = at::empty({(int64_t)maxTiles * 128, d}, h.options());
+        chronos::launch_hy_moe_glu_grouped((const uint16_t*)h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(),
+                                           (const uint16_t*)w_gu.data_ptr(), (const uint16_t*)w_down.data_ptr(),
+                                           (uint16_t*)out.data_ptr(), meta.data_ptr<int32_t>(), (uint16_t*)z.data_ptr(),
+                                           (uint16_t*)yrows.data_ptr(), (int)T, (int)d, (int)F, (int)E, top, (float)limit,
+                                           (float)slope, (float)shift, stream());
+        return out;
+    }
+    need((2 * d + 2 * F) * 4 <= 160 * 1024, "moe_glu_ffn: a token's rows must fit the LDS");
     chronos::launch_hy_moe_glu_token(h.data_ptr(), idx.data_ptr<int32_t>(), wt.data_ptr<float>(), w_gu.data_ptr(),
                                      w_down.data_ptr(), out.data_ptr(), (int)T, (int)d, (int)F, (int)E, (int)idx.size(1),
-                                     (float)limit, (float)slope, (float)shift, f32(h), stream());
+                                     (float)limit, (float)slope, (float)shift, tiled, f32(h), stream());
     return out;
 }
 
@@ -533,7 +551,7 @@ TORCH_LIBRARY_FRAGMENT(chronos, m) {
           "int Dv) -> Tensor");
     m.def("hy_moe_route_topk(Tensor h, Tensor w, Tensor bias, int top) -> (Tensor, Tensor)");
     m.def("hy_moe_glu_ffn(Tensor h, Tensor idx, Tensor wt, Tensor w_gu, Tensor w_down, float limit, float slope, "
-          "float shift) -> Tensor");
+          "float shift, bool tiled) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(chronos, CUDA, m) {

@@ -6,12 +6,13 @@
 //                 are zero when the step starts at position 0.  A second launch then rewrites the history.
 //   delta_prep    per token: 1 / |q|, 1 / |k| per query/key head (float), decay = exp(-exp(A) softplus(a)) and
 //                 beta = sigmoid(b) per value head.
-//   linear_scan   per (sequence, value head, 64 value columns per wave): the state's column lives in registers (lane =
-//                 column, all D rows), tokens are staged 16 at a time in LDS (scaled q and k rows in float, the
-//                 decays, the values), and every token does
+//   linear_scan   per (sequence, value head, 64 value columns): the state lives in registers (a wave owns 16 columns,
+//                 a lane one column's quarter of the D rows), tokens are staged 16 at a time in LDS (q and k rows in
+//                 float, the decays, the values) with the next stage's loads in flight, and every token does
 //                     S <- decay * S;  u = v - S^T k (times beta; delta rule only, else u = v);  S <- S + k u^T;
 //                     o = S^T q
-//                 with no cross-lane traffic.  decay is one number per head or one per state row.  The same kernel
+//                 with two 2-step cross-lane sums (S^T k and S^T q over the four row groups).  decay is one number per
+//                 head or one per state row.  The same kernel
 //                 serves prompt portions of any length and decode rows (a range of one token); a range that starts at
 //                 position 0 starts from the zero state, so a reused slot needs no clearing.
 #include "hybrid_common.h"
@@ -99,105 +100,148 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(const T* __restrict__ y
 }
 
 constexpr int kScanTC = 16;  // tokens per LDS stage
+constexpr int kScanRG = 4;   // row groups per wave: lane = 16 columns x 4 groups of DP / 4 state rows
+constexpr int kScanCW = 64 / kScanRG;
 
-// LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64 NW] | scalar decay [TC] | beta [TC]
+template <typename T> __device__ __forceinline__ T zero_of();
+template <> __device__ __forceinline__ float zero_of<float>() { return 0.f; }
+template <> __device__ __forceinline__ uint16_t zero_of<uint16_t>() { return 0; }
+
+// 256 threads: wave w owns value columns 16 w .. 16 w + 15 of the workgroup's 64; a lane holds DP / 4 rows of one
+// column.  LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64] | per token: decay, beta,
+// q scale, k scale.  The next stage's global loads are issued before the current stage's tokens are processed and
+// land in LDS afterwards, so the token loop never waits on global memory; the scales of q and k are folded into
+// per-token scalars (S^T k_hat = s_k S^T k, k_hat u^T = k (s_k u)^T, S^T q_hat = s_q S^T q).
 template <typename T, int DP, bool DELTA, bool CHD>
 __global__ void __launch_bounds__(256) linear_scan_kernel(
         const T* __restrict__ proj, int ldp, int q_off, int k_off, int v_off, const float* __restrict__ qscale,
         const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, const float* __restrict__ beta,
         const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots,
         float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv) {
-    extern __shared__ __attribute__((aligned(16))) float ls_smem[];
-    constexpr int TC = kScanTC;
-    const int NW = blockDim.x >> 6;
-    float* qs = ls_smem;
-    float* ks = qs + TC * DP;
-    float* ds = ks + TC * DP;
-    float* vs = ds + (CHD ? TC * DP : 0);
-    float* gs = vs + TC * 64 * NW;
-    float* bs = gs + TC;
+    constexpr int TC = kScanTC, RG = kScanRG, CW = kScanCW, RL = DP / RG, NE = TC * DP / 256;
+    __shared__ __attribute__((aligned(16))) float qs[TC * DP];
+    __shared__ __attribute__((aligned(16))) float ks[TC * DP];
+    __shared__ __attribute__((aligned(16))) float ds[CHD ? TC * DP : 4];
+    __shared__ float vs[TC * 64];
+    __shared__ float gs[TC], bs[TC], qsc[TC], ksc[TC];
     const int b = blockIdx.x, hd = blockIdx.y;
     const int t0 = q_start[b], t1 = q_start[b + 1];
     if (t1 <= t0) return;
     const int hk = hd / (H / HK);
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int col0 = blockIdx.z * 64 * NW;
-    const int col = col0 + wv * 64 + lane;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, rg = lane / CW, c = lane % CW;
+    const int col0 = blockIdx.z * 64;
+    const int col = col0 + wv * CW + c;
     const bool live = col < Dv;
     float* Sp = S + (((int64_t)slots[b] * H + hd) * D) * Dv + col;
-    float st_[DP];
+    float st_[RL];
     if (pos0[b] > 0 && live) {
 #pragma unroll
-        for (int r = 0; r < DP; ++r) st_[r] = r < D ? Sp[(int64_t)r * Dv] : 0.f;
+        for (int i = 0; i < RL; ++i) st_[i] = rg * RL + i < D ? Sp[(int64_t)(rg * RL + i) * Dv] : 0.f;
     } else {
 #pragma unroll
-        for (int r = 0; r < DP; ++r) st_[r] = 0.f;
+        for (int i = 0; i < RL; ++i) st_[i] = 0.f;
     }
+    // staging registers of one stage: element e of thread x is (token e' = (x + 256 e) / DP, row (x + 256 e) % DP)
+    T qraw[NE], kraw[NE], vraw[4];
+    float draw[CHD ? NE : 1], sraw[4];
+    auto fetch = [&](int tb) {
+        const int nt = min(TC, t1 - tb);
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int i = threadIdx.x + 256 * e, tt = i / DP, r = i % DP;
+            const bool ok = tt < nt && r < D;
+            const int64_t t = tb + tt;
+            qraw[e] = ok ? proj[t * ldp + q_off + hk * D + r] : zero_of<T>();
+            kraw[e] = ok ? proj[t * ldp + k_off + hk * D + r] : zero_of<T>();
+            if constexpr (CHD) draw[e] = ok ? decay[(t * H + hd) * D + r] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = threadIdx.x + 256 * e, tt = i >> 6, cc = col0 + (i & 63);
+            vraw[e] = (tt < nt && cc < Dv) ? proj[(int64_t)(tb + tt) * ldp + v_off + hd * Dv + cc] : zero_of<T>();
+        }
+        if (threadIdx.x < TC) {
+            const bool ok = (int)threadIdx.x < nt;
+            const int64_t t = tb + threadIdx.x;
+            sraw[0] = (!CHD && ok) ? decay[t * H + hd] : 1.f;
+            sraw[1] = (DELTA && ok) ? beta[t * H + hd] : 0.f;
+            sraw[2] = (qscale != nullptr && ok) ? qscale[t * HK + hk] : q_mul;
+            sraw[3] = (kscale != nullptr && ok) ? kscale[t * HK + hk] : 1.f;
+        }
+    };
+    auto land = [&]() {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int i = threadIdx.x + 256 * e;
+            qs[i] = ld<T>(&qraw[e]);
+            ks[i] = ld<T>(&kraw[e]);
+            if constexpr (CHD) ds[i] = draw[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vs[threadIdx.x + 256 * e] = ld<T>(&vraw[e]);
+        if (threadIdx.x < TC) {
+            gs[threadIdx.x] = sraw[0];
+            bs[threadIdx.x] = sraw[1];
+            qsc[threadIdx.x] = sraw[2];
+            ksc[threadIdx.x] = sraw[3];
+        }
+    };
+    fetch(t0);
     for (int tb = t0; tb < t1; tb += TC) {
         const int nt = min(TC, t1 - tb);
         __syncthreads();  // the previous stage has been consumed
-        for (int i = threadIdx.x; i < nt * DP; i += blockDim.x) {
-            const int tt = i / DP, r = i % DP;
-            const int64_t t = tb + tt;
-            float qv = 0.f, kv = 0.f;
-            if (r < D) {
-                qv = ld<T>(proj + t * ldp + q_off + hk * D + r) * (qscale != nullptr ? qscale[t * HK + hk] : q_mul);
-                kv = ld<T>(proj + t * ldp + k_off + hk * D + r) * (kscale != nullptr ? kscale[t * HK + hk] : 1.f);
-            }
-            qs[i] = qv;
-            ks[i] = kv;
-            if constexpr (CHD) ds[i] = r < D ? decay[(t * H + hd) * D + r] : 0.f;
-        }
-        for (int i = threadIdx.x; i < nt * 64 * NW; i += blockDim.x) {
-            const int tt = i / (64 * NW), c = col0 + i % (64 * NW);
-            vs[i] = c < Dv ? ld<T>(proj + (int64_t)(tb + tt) * ldp + v_off + hd * Dv + c) : 0.f;
-        }
-        if (threadIdx.x < nt) {
-            if constexpr (!CHD) gs[threadIdx.x] = decay[(int64_t)(tb + threadIdx.x) * H + hd];
-            if constexpr (DELTA) bs[threadIdx.x] = beta[(int64_t)(tb + threadIdx.x) * H + hd];
-        }
+        land();
         __syncthreads();
+        if (tb + TC < t1) fetch(tb + TC);
         for (int tt = 0; tt < nt; ++tt) {
-            const f32x4* q4 = reinterpret_cast<const f32x4*>(qs + tt * DP);
-            const f32x4* k4 = reinterpret_cast<const f32x4*>(ks + tt * DP);
-            const f32x4* d4 = reinterpret_cast<const f32x4*>(ds + tt * DP);
+            const f32x4* q4 = reinterpret_cast<const f32x4*>(qs + tt * DP + rg * RL);
+            const f32x4* k4 = reinterpret_cast<const f32x4*>(ks + tt * DP + rg * RL);
             float g = 1.f;
             if constexpr (CHD) {
+                const f32x4* d4 = reinterpret_cast<const f32x4*>(ds + tt * DP + rg * RL);
 #pragma unroll
-                for (int r = 0; r < DP; r += 4) {
-                    const f32x4 dv = d4[r >> 2];
-                    st_[r] *= dv[0]; st_[r + 1] *= dv[1]; st_[r + 2] *= dv[2]; st_[r + 3] *= dv[3];
+                for (int i = 0; i < RL; i += 4) {
+                    const f32x4 dv = d4[i >> 2];
+                    st_[i] *= dv[0]; st_[i + 1] *= dv[1]; st_[i + 2] *= dv[2]; st_[i + 3] *= dv[3];
                 }
             } else {
                 g = gs[tt];
             }
-            float u = vs[tt * 64 * NW + wv * 64 + lane];
+            const float sk = ksc[tt];
+            float u = vs[tt * 64 + wv * CW + c];
             if constexpr (DELTA) {
                 float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
-                for (int r = 0; r < DP; r += 4) {
-                    const f32x4 kv = k4[r >> 2];
-                    p0 += st_[r] * kv[0]; p1 += st_[r + 1] * kv[1]; p2 += st_[r + 2] * kv[2]; p3 += st_[r + 3] * kv[3];
+                for (int i = 0; i < RL; i += 4) {
+                    const f32x4 kv = k4[i >> 2];
+                    p0 += st_[i] * kv[0]; p1 += st_[i + 1] * kv[1]; p2 += st_[i + 2] * kv[2]; p3 += st_[i + 3] * kv[3];
                 }
-                u = bs[tt] * (u - g * ((p0 + p1) + (p2 + p3)));
+                float p = (p0 + p1) + (p2 + p3);
+                p += __shfl_xor(p, 16, 64);
+                p += __shfl_xor(p, 32, 64);
+                u = bs[tt] * (u - g * sk * p);
             }
+            const float uk = u * sk;
             float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
-            for (int r = 0; r < DP; r += 4) {
-                const f32x4 kv = k4[r >> 2], qv = q4[r >> 2];
-                st_[r] = g * st_[r] + kv[0] * u;
-                st_[r + 1] = g * st_[r + 1] + kv[1] * u;
-                st_[r + 2] = g * st_[r + 2] + kv[2] * u;
-                st_[r + 3] = g * st_[r + 3] + kv[3] * u;
-                a0 += st_[r] * qv[0]; a1 += st_[r + 1] * qv[1]; a2 += st_[r + 2] * qv[2]; a3 += st_[r + 3] * qv[3];
+            for (int i = 0; i < RL; i += 4) {
+                const f32x4 kv = k4[i >> 2], qv = q4[i >> 2];
+                st_[i] = g * st_[i] + kv[0] * uk;
+                st_[i + 1] = g * st_[i + 1] + kv[1] * uk;
+                st_[i + 2] = g * st_[i + 2] + kv[2] * uk;
+                st_[i + 3] = g * st_[i + 3] + kv[3] * uk;
+                a0 += st_[i] * qv[0]; a1 += st_[i + 1] * qv[1]; a2 += st_[i + 2] * qv[2]; a3 += st_[i + 3] * qv[3];
             }
-            if (live) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = (a0 + a1) + (a2 + a3);
+            float a = (a0 + a1) + (a2 + a3);
+            a += __shfl_xor(a, 16, 64);
+            a += __shfl_xor(a, 32, 64);
+            if (live && rg == 0) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = a * qsc[tt];
         }
     }
     if (live) {
 #pragma unroll
-        for (int r = 0; r < DP; ++r)
-            if (r < D) Sp[(int64_t)r * Dv] = st_[r];
+        for (int i = 0; i < RL; ++i)
+            if (rg * RL + i < D) Sp[(int64_t)(rg * RL + i) * Dv] = st_[i];
     }
 }
 
@@ -229,14 +273,9 @@ static void linear_scan_launch(const T* proj, int ldp, int q_off, int k_off, int
                                const float* kscale, float q_mul, const float* decay, const float* beta,
                                const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
                                int HK, int H, int D, int Dv, hipStream_t s) {
-    const int NW = Dv > 192 ? 4 : Dv > 128 ? 3 : Dv > 64 ? 2 : 1;
-    const int bytes = (hy::kScanTC * DP * (CHD ? 3 : 2) + hy::kScanTC * 64 * NW + 2 * hy::kScanTC) * 4;
-    auto kern = hy::linear_scan_kernel<T, DP, DELTA, CHD>;
-    if (bytes > 48 * 1024)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    const dim3 grid(B, H, (Dv + 64 * NW - 1) / (64 * NW));
-    kern<<<grid, 64 * NW, bytes, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0,
-                                      slots, S, o, HK, H, D, Dv);
+    const dim3 grid(B, H, (Dv + 63) / 64);
+    hy::linear_scan_kernel<T, DP, DELTA, CHD><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
+                                                                  beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
 }
 
 template <typename T, bool DELTA, bool CHD>

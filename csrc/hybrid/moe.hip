@@ -167,13 +167,14 @@ __global__ void __launch_bounds__(256) moe_select_topk_kernel(const float* __res
 }
 
 // Gated experts: per token sum_k weight_k * W_down,e ( g sigmoid(slope g) (u + shift) ), g = min(W_gate,e h, limit),
-// u = clamp(W_up,e h, +-limit).  w_gu [E, 2F, d]: gate rows then up rows.  LDS: h (d) | gate, up (2F) | out (d).
+// u = clamp(W_up,e h, +-limit).  w_gu [E, 2F, d]: gate rows then up rows, or (tiled) in the grouped path's tile order.
+// LDS: h (d) | gate, up (2F) | out (d).
 template <typename T>
 __global__ void __launch_bounds__(256) moe_glu_token_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
                                                             const float* __restrict__ wt, const T* __restrict__ w_gu,
                                                             const T* __restrict__ w_down, T* __restrict__ out, int d,
                                                             int F, int E, int top, float limit, float slope,
-                                                            float shift) {
+                                                            float shift, int tiled) {
     extern __shared__ float sm[];
     float* hs = sm;
     float* zs = hs + d;
@@ -191,7 +192,12 @@ __global__ void __launch_bounds__(256) moe_glu_token_kernel(const T* __restrict_
         if (e < 0 || e >= E) continue;  // (uniform over the workgroup)
         const T* wu = w_gu + (int64_t)e * 2 * F * d;
         for (int f = wv; f < 2 * F; f += 4) {
-            const T* wr = wu + (int64_t)f * d;
+            int row = f;
+            if (tiled) {  // the grouped path's row order: per 128-row tile and 64-row half, 32 gate rows then their up rows
+                const int c = f < F ? f : f - F;
+                row = (c >> 6) * 128 + ((c >> 5) & 1) * 64 + (c & 31) + (f < F ? 0 : 32);
+            }
+            const T* wr = wu + (int64_t)row * d;
             float acc = 0.f;
             for (int i = lane; i < d; i += 64) acc += ld<T>(wr + i) * hs[i];
             acc = wave_sum(acc);
@@ -253,17 +259,17 @@ void launch_hy_moe_route_topk(const void* h, const void* w, const float* bias, f
 
 void launch_hy_moe_glu_token(const void* h, const int32_t* idx, const float* wt, const void* w_gu, const void* w_down,
                              void* out, int T, int d, int F, int E, int top, float limit, float slope, float shift,
-                             bool f32, hipStream_t s) {
+                             bool tiled, bool f32, hipStream_t s) {
     if (T == 0) return;
     const int bytes = (2 * d + 2 * F) * 4;
     if (f32) {
         auto kern = hy::moe_glu_token_kernel<float>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<T, 256, bytes, s>>>((const float*)h, idx, wt, (const float*)w_gu, (const float*)w_down, (float*)out, d, F, E, top, limit, slope, shift);
+        kern<<<T, 256, bytes, s>>>((const float*)h, idx, wt, (const float*)w_gu, (const float*)w_down, (float*)out, d, F, E, top, limit, slope, shift, tiled);
     } else {
         auto kern = hy::moe_glu_token_kernel<uint16_t>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<T, 256, bytes, s>>>((const uint16_t*)h, idx, wt, (const uint16_t*)w_gu, (const uint16_t*)w_down, (uint16_t*)out, d, F, E, top, limit, slope, shift);
+        kern<<<T, 256, bytes, s>>>((const uint16_t*)h, idx, wt, (const uint16_t*)w_gu, (const uint16_t*)w_down, (uint16_t*)out, d, F, E, top, limit, slope, shift, tiled);
     }
 }
 

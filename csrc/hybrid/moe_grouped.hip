@@ -12,6 +12,10 @@
 //   combine   out[t, :] = sum_k weight[t, k] * Y[row(t, k), :]  (+ weight * h[t, :] for an identity expert), summed
 //             in the order of k in float: the result does not depend on what else is in the batch.
 //
+// Gated experts (act = gated unit): the up GEMM runs over W_gu [E, 2F, d] whose rows are PERMUTED at weight-packing
+// time (moe_glu_row_order) so that every 128-row tile holds 64 gate rows and their 64 up rows in the accumulator
+// positions of the same lane; the epilogue combines them and writes 64 columns of Z [rows, F] per tile.
+//
 // The tile loop is the 128 x 128 x 64 LDS-DMA ring of csrc/kernels/gemm.hip (4 waves as 2 x 2, 16x16x32 bf16 MFMAs,
 // XOR-swizzled images, one barrier per k-step with a counted vmcnt).  Needs d % 128 == 0 and F % 128 == 0.
 #include "hybrid_common.h"
@@ -80,11 +84,14 @@ __global__ void __launch_bounds__(1024) moe_align_kernel(const int32_t* __restri
 }
 
 // y[row, n] = sum_k x[src(row), k] * w[e][n, k]; GATHER: src(row) = row_item[row] / top (rows of h), else row.
-// ACT >= 0: activation of that kind in the epilogue.
+// ACT >= 0: activation of that kind in the epilogue.  ACT == kActGlu: w holds N = 2F permuted gate / up rows, y is
+// [rows, N / 2], and (limit, slope, shift) are the gated unit's constants.
+constexpr int kActGlu = 2;
 template <bool GATHER, int ACT>
 __global__ void __launch_bounds__(256) moe_gemm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                        uint16_t* __restrict__ y, const int32_t* __restrict__ meta,
-                                                       int maxTiles, int top, int N, int K) {
+                                                       int maxTiles, int top, int N, int K, float limit, float slope,
+                                                       float shift) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     const int nt = N / GBN;
     const int tile = blockIdx.x / nt, tn = blockIdx.x % nt;
@@ -156,13 +163,29 @@ __global__ void __launch_bounds__(256) moe_gemm_kernel(const uint16_t* __restric
     for (int t = 0; t < 4; ++t) {
         const int m = m0 + 64 * wm + 16 * t + (lane & 15);
         if (row_item[m] < 0) continue;
+        if constexpr (ACT == kActGlu) {
+            // tile-local rows 64 wn + 16 s + j: s = 0, 1 are gate rows, s = 2, 3 the up rows of the same outputs
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                u16x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float a = fminf(bf2f(f2bf(acc[s][t][i])), limit);
+                    const float u = fminf(fmaxf(bf2f(f2bf(acc[s + 2][t][i])), -limit), limit);
+                    o[i] = f2bf(a * sigmoidf_(slope * a) * (u + shift));
+                }
+                const int n = tn * 64 + 32 * wn + 16 * s + 4 * (lane >> 4);
+                *reinterpret_cast<u16x4*>(y + (int64_t)m * (N / 2) + n) = o;
+            }
+            continue;
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             u16x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float v = acc[s][t][i];
-                if constexpr (ACT >= 0) v = act_apply(bf2f(f2bf(v)), ACT);
+                if constexpr (ACT >= 0 && ACT != kActGlu) v = act_apply(bf2f(f2bf(v)), ACT);
                 o[i] = f2bf(v);
             }
             const int n = tn * GBN + 64 * wn + 16 * s + 4 * (lane >> 4);
@@ -212,9 +235,29 @@ void launch_hy_moe_grouped(const uint16_t* h, const int32_t* idx, const float* w
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(hy::moe_gemm_kernel<false, -1>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         attr = true;
     }
-    if (act == 0) hy::moe_gemm_kernel<true, 0><<<maxTiles * (F / hy::GBN), 256, lds, s>>>(h, w_up, z, meta, maxTiles, top, F, d);
-    else hy::moe_gemm_kernel<true, 1><<<maxTiles * (F / hy::GBN), 256, lds, s>>>(h, w_up, z, meta, maxTiles, top, F, d);
-    hy::moe_gemm_kernel<false, -1><<<maxTiles * (d / hy::GBN), 256, lds, s>>>(z, w_down, yrows, meta, maxTiles, top, d, F);
+    if (act == 0) hy::moe_gemm_kernel<true, 0><<<maxTiles * (F / hy::GBN), 256, lds, s>>>(h, w_up, z, meta, maxTiles, top, F, d, 0.f, 0.f, 0.f);
+    else hy::moe_gemm_kernel<true, 1><<<maxTiles * (F / hy::GBN), 256, lds, s>>>(h, w_up, z, meta, maxTiles, top, F, d, 0.f, 0.f, 0.f);
+    hy::moe_gemm_kernel<false, -1><<<maxTiles * (d / hy::GBN), 256, lds, s>>>(z, w_down, yrows, meta, maxTiles, top, d, F, 0.f, 0.f, 0.f);
+    hy::moe_combine_kernel<<<T, 256, 0, s>>>(h, yrows, idx, wt, meta + 1 + maxTiles + maxTiles * hy::GBM, out, d, top, E);
+}
+
+// Gated experts.  w_gu: bf16 [E, 2F, d] in the tile order of moe_glu_row_order; z: bf16 [maxTiles * 128, F];
+// needs d % 128 == 0 and F % 128 == 0 (the down GEMM's k-steps and the up GEMM's 64-output tiles).
+void launch_hy_moe_glu_grouped(const uint16_t* h, const int32_t* idx, const float* wt, const uint16_t* w_gu,
+                               const uint16_t* w_down, uint16_t* out, int32_t* meta, uint16_t* z, uint16_t* yrows, int T,
+                               int d, int F, int E, int top, float limit, float slope, float shift, hipStream_t s) {
+    if (T == 0) return;
+    const int items = T * top, maxTiles = hy_moe_max_tiles(items, E);
+    hy::moe_align_kernel<<<1, 1024, 0, s>>>(idx, items, E, maxTiles, meta);
+    const int lds = hy::GSTAGES * 2 * hy::kImg;
+    static bool attr = false;
+    if (!attr) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(hy::moe_gemm_kernel<true, hy::kActGlu>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(hy::moe_gemm_kernel<false, -1>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        attr = true;
+    }
+    hy::moe_gemm_kernel<true, hy::kActGlu><<<maxTiles * (2 * F / hy::GBN), 256, lds, s>>>(h, w_gu, z, meta, maxTiles, top, 2 * F, d, limit, slope, shift);
+    hy::moe_gemm_kernel<false, -1><<<maxTiles * (d / hy::GBN), 256, lds, s>>>(z, w_down, yrows, meta, maxTiles, top, d, F, 0.f, 0.f, 0.f);
     hy::moe_combine_kernel<<<T, 256, 0, s>>>(h, yrows, idx, wt, meta + 1 + maxTiles + maxTiles * hy::GBM, out, d, top, E);
 }
 

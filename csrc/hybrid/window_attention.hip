@@ -84,7 +84,8 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
         const T* __restrict__ qkv, int ldq, const T* __restrict__ kc, const T* __restrict__ vc,
         const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
         const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
-        T* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int QT) {
+        T* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int QT,
+        int rows_cap) {
     extern __shared__ __attribute__((aligned(16))) unsigned char wa_smem[];
     constexpr int PAD = WaPad<T>::V;
     const int R = H / G;
@@ -97,7 +98,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
     T* Ks = reinterpret_cast<T*>(wa_smem);
     T* Vs = Ks + kWaKT * ldk;
     float* Qs = reinterpret_cast<float*>(wa_smem + (((size_t)kWaKT * (ldk + ldv) * sizeof(T) + 15) & ~(size_t)15));
-    float* Ps = Qs + (size_t)kWaRows * D;
+    float* Ps = Qs + (size_t)rows_cap * D;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     float* Pw = Ps + wv * kWaRB * kWaKT;
     for (int i = threadIdx.x; i < rows * D; i += 256) {
@@ -232,30 +233,48 @@ void launch_hy_window_prep(void* qkv, int ld, int H, int G, int D, int Dv, const
     else hy::window_prep_kernel<uint16_t><<<T, 256, bytes, s>>>((uint16_t*)qkv, ld, H, G, D, Dv, (const uint16_t*)v_first, lam, pos, tok_seq, block_table, max_blocks, q_norm, k_norm, eps, cos_sin, dims, (uint16_t*)kc, (uint16_t*)vc, BS, (uint16_t*)v_out);
 }
 
-// LDS bytes of the general kernel; the caller checks it against the 160 KB of a CU.
-size_t hy_window_attention_lds(int D, int Dv, bool f32) {
+// LDS bytes of the general kernel with room for `rows` (token, head) query rows.
+static size_t window_attention_lds(int rows, int D, int Dv, bool f32) {
     const size_t e = f32 ? 4 : 2, pad = f32 ? 1 : 2;
     const size_t tiles = ((size_t)hy::kWaKT * (D + pad + Dv + pad) * e + 15) & ~(size_t)15;
-    return tiles + ((size_t)hy::kWaRows * D + 4 * hy::kWaRB * hy::kWaKT) * 4;
+    return tiles + ((size_t)rows * D + 4 * hy::kWaRB * hy::kWaKT) * 4;
 }
 
+// Query rows per workgroup of the general kernel: the most (64 at most, a power of two, at least the R heads of a
+// group) whose float copies fit the 160 KB of a CU beside a key tile; 0: these sizes do not fit at all.
+int hy_window_rows_cap(int R, int D, int Dv, bool f32) {
+    for (int rows = hy::kWaRows; rows >= 1 && rows >= R; rows >>= 1)
+        if (window_attention_lds(rows, D, Dv, f32) <= 160 * 1024) return rows;
+    return 0;
+}
+
+bool launch_hy_window_attention_mfma(const uint16_t*, int, const uint16_t*, const uint16_t*, const int32_t*, int,
+                                     const int32_t*, const int32_t*, const float*, const float*, uint16_t*, int, int, int,
+                                     int, int, int, int, float, int, int, hipStream_t);
+
+// bfloat16 at matrix-core sizes runs window_attention_mfma.hip; float32 and every other size the general kernel.
 void launch_hy_window_attention(const void* qkv, int ld, const void* kc, const void* vc, const int32_t* block_table,
                                 int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
                                 const float* gate, void* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
                                 float scale, int window, int keep, bool f32, hipStream_t s) {
     if (B == 0 || max_q == 0) return;
-    const int bytes = (int)hy_window_attention_lds(D, Dv, f32);
-    const int R = H / G;   // the caller has checked R <= 64, Dv <= 256 and the LDS size
-    const int QT = std::max(1, std::min(hy::kWaQT, hy::kWaRows / R));
+    if (!f32 && launch_hy_window_attention_mfma((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc,
+                                                block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, B,
+                                                max_q, H, G, D, Dv, BS, scale, window, keep, s))
+        return;
+    const int R = H / G;   // the caller has checked R <= 64, Dv <= 256 and that hy_window_rows_cap is not 0
+    const int rows_cap = hy_window_rows_cap(R, D, Dv, f32);
+    const int bytes = (int)window_attention_lds(rows_cap, D, Dv, f32);
+    const int QT = std::max(1, std::min(hy::kWaQT, rows_cap / R));
     const dim3 grid(B, (max_q + QT - 1) / QT, G);
     if (f32) {
         auto kern = hy::window_attention_kernel<float>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<grid, 256, bytes, s>>>((const float*)qkv, ld, (const float*)kc, (const float*)vc, block_table, max_blocks, q_start, pos, sink, gate, (float*)out, H, G, D, Dv, BS, scale, window, keep, QT);
+        kern<<<grid, 256, bytes, s>>>((const float*)qkv, ld, (const float*)kc, (const float*)vc, block_table, max_blocks, q_start, pos, sink, gate, (float*)out, H, G, D, Dv, BS, scale, window, keep, QT, rows_cap);
     } else {
         auto kern = hy::window_attention_kernel<uint16_t>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<grid, 256, bytes, s>>>((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc, block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, H, G, D, Dv, BS, scale, window, keep, QT);
+        kern<<<grid, 256, bytes, s>>>((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc, block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, H, G, D, Dv, BS, scale, window, keep, QT, rows_cap);
     }
 }
 

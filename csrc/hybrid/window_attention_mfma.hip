@@ -1,0 +1,229 @@
+// window_attention_mfma.hip — the bfloat16 windowed sink attention on the matrix cores (see window_attention.hip for
+// the math and the visible set).
+//
+// One workgroup takes one sequence, one key/value head and 16 NW (token, head-of-the-group) rows — 16 per wave; rows
+// are (token * R + head within the group), so any group size tiles the same way — and walks the keys it can see 64
+// at a time: first the kept first tokens that lie below the window's first tile, then the tiles from the window's
+// first key to the last query.  Per tile:
+//   * the keys are staged row-major [64][D] and the values transposed [Dv][64] in LDS (both MFMA operands want 8
+//     consecutive k-values per lane: dims for the scores, KEYS for the sum); the transposed image is written as
+//     32-bit words holding two neighbouring keys;
+//   * scores  S^T = K Q^T : 16x16x32 MFMAs, key rows as A operand, the wave's 16 query rows (in registers for the
+//     whole kernel) as B operand: a lane ends up with 4 keys x 1 query row per 16-key tile;
+//   * softmax in float per query row (lane & 15): each row masks by its own position (causal, window, kept tokens),
+//     running maximum and sum, reductions over the 4 lane groups by two shuffles;
+//   * sum  O^T = V^T P^T : the lane's 8 weights of two neighbouring 16-key tiles ARE a B operand (the k index is a
+//     fixed permutation of the 32 keys, the same one the transposed value image is read with); each weight enters
+//     as two bfloat16 terms (rounded value + remainder), which keeps the float softmax weights nearly exact.
+// After the last tile the head's sink joins the denominator and the row is scaled by sigmoid(gate).
+// Sizes: D % 32 == 0, Dv % 16 == 0, D <= 256, Dv <= 256.  Everything else takes the general kernel.
+#include "hybrid_common.h"
+
+namespace chronos {
+namespace hy {
+
+constexpr int WKT = 64;  // keys per tile
+
+template <int NS, int NCT, int NW>
+__global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
+        const uint16_t* __restrict__ qkv, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+        const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
+        const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
+        uint16_t* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int KT = WKT, NT = 64 * NW, RPB = 16 * NW, PP = KT / 2;
+    const int R = H / G;
+    const int b = blockIdx.x, kvh = blockIdx.z;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    const int rows_total = (t1 - t0) * R;
+    const int rb0 = blockIdx.y * RPB;
+    if (rb0 >= rows_total) return;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, g4 = lane >> 4, qi = lane & 15;
+    const int ns = D / 32, nct = Dv / 16;
+    const int krs = D * 2 + 16;          // row-major key image: bytes per key row
+    constexpr int vts = KT * 2 + 8;      // transposed value image: bytes per value column
+    __shared__ int krow[KT];             // cache row (page * page size + slot) of each key of the tile
+    unsigned char* kimg = smem;
+    unsigned char* vimg = smem + KT * krs;
+    const int r = rb0 + wv * 16 + qi;
+    const bool rok = r < rows_total;
+    const int rc = rok ? r : rows_total - 1;
+    const int64_t tok = t0 + rc / R;
+    const int head = kvh * R + rc % R;
+    const int prow = rok ? pos[tok] : -1;
+    const int last_row = min(rows_total, rb0 + RPB) - 1;
+    const int pmin = pos[t0 + rb0 / R], pmax = pos[t0 + last_row / R];  // positions grow along the sequence
+    bf16x8 qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        if (s < ns) qf[s] = *reinterpret_cast<const bf16x8*>(qkv + tok * ldq + head * D + 32 * s + 8 * g4);
+    f32x4 O[NCT];
+#pragma unroll
+    for (int c = 0; c < NCT; ++c) O[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mrow = -INFINITY, lrow = 0.f;
+    const int32_t* bt = block_table + (int64_t)b * max_blocks;
+    const int kchunks = D / 8, vchunks = Dv / 8;
+    const int w_lo = window > 0 ? max(0, pmin - window + 1) : 0;
+    const int w_start = w_lo / KT * KT;
+    // kept first tokens below the window's first tile are keys [0, k_end); those from w_start on pass the window
+    // tiles' own test, so no key is counted twice
+    const int k_end = window > 0 ? min(keep, w_start) : 0;
+    const int n_keep_tiles = (k_end + KT - 1) / KT;
+    const int n_tiles = n_keep_tiles + (pmax - w_start) / KT + 1;
+    for (int ti = 0; ti < n_tiles; ++ti) {
+        const bool kept = ti < n_keep_tiles;
+        const int k0 = kept ? ti * KT : w_start + (ti - n_keep_tiles) * KT;
+        const int k_last = kept ? k_end - 1 : pmax;  // last real key this tile may hold
+        __syncthreads();
+        if (threadIdx.x < KT) {
+            const int key = min(k0 + (int)threadIdx.x, k_last);  // past the end: a real row, masked below
+            krow[threadIdx.x] = (bt[key / BS] * BS + key % BS) * G + kvh;
+        }
+        __syncthreads();
+        // ---- stage: work item = (key pair jp, 8-element chunk dc); lanes of a wave take consecutive key pairs
+        for (int it = threadIdx.x; it < PP * kchunks; it += NT) {
+            const int jp = it & (PP - 1), dc = it / PP;
+            const u16x8 va = *reinterpret_cast<const u16x8*>(kc + (int64_t)krow[2 * jp] * D + dc * 8);
+            const u16x8 vb = *reinterpret_cast<const u16x8*>(kc + (int64_t)krow[2 * jp + 1] * D + dc * 8);
+            *reinterpret_cast<u16x8*>(kimg + (2 * jp) * krs + dc * 16) = va;
+            *reinterpret_cast<u16x8*>(kimg + (2 * jp + 1) * krs + dc * 16) = vb;
+        }
+        for (int it = threadIdx.x; it < PP * vchunks; it += NT) {
+            const int jp = it & (PP - 1), dc = it / PP;
+            const u16x8 va = *reinterpret_cast<const u16x8*>(vc + (int64_t)krow[2 * jp] * Dv + dc * 8);
+            const u16x8 vb = *reinterpret_cast<const u16x8*>(vc + (int64_t)krow[2 * jp + 1] * Dv + dc * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                *reinterpret_cast<uint32_t*>(vimg + (dc * 8 + e) * vts + jp * 4) = (uint32_t)va[e] | ((uint32_t)vb[e] << 16);
+        }
+        __syncthreads();
+        // ---- scores: 4 key tiles of 16; lane gets keys 16 kt + 4 g4 + i of query row qi
+        constexpr int NKT = KT / 16;
+        f32x4 S[NKT];
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt) {
+            S[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const unsigned char* arow = kimg + (16 * kt + qi) * krs + g4 * 16;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                if (s < ns)
+                    S[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(arow + s * 64), qf[s],
+                                                                    S[kt], 0, 0, 0);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + 16 * kt + 4 * g4 + i;
+                const bool vis = key <= k_last && key <= prow && (window <= 0 || prow - key < window || key < keep);
+                const float sv = vis ? S[kt][i] * scale : -INFINITY;
+                S[kt][i] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(mrow, mx);
+        const float corr = (mn == -INFINITY) ? 1.f : __expf(mrow - mn);
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = (mn == -INFINITY) ? 0.f : __expf(S[kt][i] - mn);
+                S[kt][i] = p;
+                sum += p;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        lrow = lrow * corr + sum;
+        mrow = mn;
+        // ---- weighted sum of the values: k index of step u = [tile 2u keys 4g4..4g4+3 | tile 2u+1 keys 4g4..4g4+3]
+        constexpr int NU = KT / 32;
+        // the float weights enter the MFMA as a sum of two bfloat16 terms (the rounded weight and the rounding's
+        // remainder), so the weighted sum sees them to about 2^-17 instead of 2^-9
+        bf16x8 pf[NU], pl[NU];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float w = S[2 * u + (e >> 2)][e & 3];
+                const __bf16 hi = (__bf16)w;
+                pf[u][e] = hi;
+                pl[u][e] = (__bf16)(w - (float)hi);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NCT; ++c) {
+            if (c < nct) {
+                O[c] *= corr;
+                const unsigned char* vrow = vimg + (16 * c + qi) * vts + g4 * 8;
+#pragma unroll
+                for (int u = 0; u < NU; ++u) {
+                    const bf16x4 lo = *reinterpret_cast<const bf16x4*>(vrow + u * 64);
+                    const bf16x4 hi = *reinterpret_cast<const bf16x4*>(vrow + u * 64 + 32);
+                    const bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    O[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], O[c], 0, 0, 0);
+                    O[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[u], O[c], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!rok) return;
+    float oc = 1.f;
+    if (sink != nullptr) {
+        const float sk = sink[head];
+        const float mn = fmaxf(mrow, sk);
+        oc = mrow == -INFINITY ? 0.f : expf(mrow - mn);
+        lrow = lrow * oc + expf(sk - mn);
+    }
+    float f = lrow > 0.f ? oc / lrow : 0.f;
+    if (gate != nullptr) f *= sigmoidf_(gate[tok * H + head]);
+    // lane holds O^T[col = 16 c + 4 g4 + i][query row qi]
+#pragma unroll
+    for (int c = 0; c < NCT; ++c)
+        if (c < nct) {
+            const u16x4 o = u16x4{f2bf(O[c][0] * f), f2bf(O[c][1] * f), f2bf(O[c][2] * f), f2bf(O[c][3] * f)};
+            *reinterpret_cast<u16x4*>(out + (tok * H + head) * Dv + 16 * c + 4 * g4) = o;
+        }
+}
+
+}  // namespace hy
+
+template <int NS, int NCT, int NW>
+static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc, const int32_t* bt,
+                           int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
+                           const float* gate, uint16_t* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
+                           float scale, int window, int keep, hipStream_t s) {
+    auto kern = hy::window_attention_mfma_kernel<NS, NCT, NW>;
+    const int bytes = hy::WKT * (D * 2 + 16) + Dv * (hy::WKT * 2 + 8);
+    static int set_bytes = 0;
+    if (bytes > set_bytes) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        set_bytes = bytes;
+    }
+    const dim3 grid(B, (max_q * (H / G) + 16 * NW - 1) / (16 * NW), G);
+    kern<<<grid, 64 * NW, bytes, s>>>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, H, G, D, Dv, BS, scale,
+                                      window, keep);
+}
+
+bool hy_window_mfma_ok(int ldq, int D, int Dv) { return !(D % 32 || Dv % 16 || D > 256 || Dv > 256 || ldq % 8); }
+
+// false: these sizes are not served here (the caller takes the general kernel).
+bool launch_hy_window_attention_mfma(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc,
+                                     const int32_t* bt, int max_blocks, const int32_t* q_start, const int32_t* pos,
+                                     const float* sink, const float* gate, uint16_t* out, int B, int max_q, int H, int G,
+                                     int D, int Dv, int BS, float scale, int window, int keep, hipStream_t s) {
+    if (!hy_window_mfma_ok(ldq, D, Dv)) return false;
+    if (B == 0 || max_q == 0) return true;
+#define HY_WAM(NS, NCT, NW) wa_mfma_launch<NS, NCT, NW>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, B, max_q, H, G, D, Dv, BS, scale, window, keep, s)
+    // 8 waves per workgroup when a sequence brings more than 64 rows per key/value head: a staged tile then serves
+    // 128 rows and every SIMD holds two waves
+    const bool nw8 = max_q * (H / G) > 64;
+    if (D <= 128 && Dv <= 128) { if (nw8) HY_WAM(4, 8, 8); else HY_WAM(4, 8, 4); }
+    else { if (nw8) HY_WAM(8, 16, 8); else HY_WAM(8, 16, 4); }
+#undef HY_WAM
+    return true;
+}
+
+}  // namespace chronos

@@ -367,9 +367,15 @@ def pack_glu(spec: GluFFSpec, t: dict, device, act_dtype) -> dict:
 def pack_moe_glu(spec: MoEGluSpec, t: dict, device, act_dtype) -> dict:
     """t: router, router.b, e<k>.gate, e<k>.up, e<k>.down.  Per expert gate rows then up rows, stacked [E, 2F, d]."""
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
-    return dict(w_router=a(t["router"]), b_router=t["router.b"].to(device=device, dtype=torch.float32).contiguous(),
-                w_gu=a(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(spec.experts)])),
-                w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
+    out = dict(w_router=a(t["router"]), b_router=t["router.b"].to(device=device, dtype=torch.float32).contiguous(),
+               w_gu=a(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(spec.experts)])),
+               w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
+    d = out["w_gu"].shape[2]
+    if act_dtype == torch.bfloat16 and torch.device(device).type == "cuda" and d % 128 == 0 and spec.ff % 128 == 0:
+        # prompt portions take the grouped matrix-core path, which wants gate and up rows interleaved per tile
+        out["w_gu"] = out["w_gu"][:, hops.moe_glu_row_order(spec.ff).to(out["w_gu"].device)].contiguous()
+        out["gu_tiled"] = True
+    return out
 
 
 def rope_cos_sin(base: float, dims: int, max_pos: int, device, scaling: Optional[tuple] = None) -> torch.Tensor:
@@ -486,7 +492,8 @@ def ff_glu(model, spec: GluFFSpec, w: dict, h):
 
 def ff_moe_glu(model, spec: MoEGluSpec, w: dict, h):
     idx, wt = hops.moe_route_topk(h, w["w_router"], w["b_router"], spec.top)
-    return hops.moe_glu_ffn(h, idx, wt, w["w_gu"], w["w_down"], spec.limit, spec.slope, spec.shift, model.act_dtype)
+    return hops.moe_glu_ffn(h, idx, wt, w["w_gu"], w["w_down"], spec.limit, spec.slope, spec.shift, model.act_dtype,
+                            bool(w.get("gu_tiled", False)))
 
 
 def ff_dense(model, spec: DenseFFSpec, w: dict, h):

@@ -215,7 +215,22 @@ def moe_route_topk(h, w_router, bias, top: int):
     return ref.moe_route_topk(h, w_router, bias, top)
 
 
-def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit: float, slope: float, shift: float, act_dtype):
+def moe_glu_row_order(F: int) -> torch.Tensor:
+    """Row order of a gated expert's [2F, d] gate-then-up matrix for the grouped MFMA path (F % 128 == 0): every
+    128-row tile holds, for each of its two 64-row halves, 32 gate rows followed by the 32 up rows of the same
+    outputs, so that a lane's accumulators hold a gate value and its up value."""
+    n = torch.arange(2 * F)
+    tile, local = n // 128, n % 128
+    half, s, j = local // 64, (local % 64) // 16, local % 16
+    out_col = tile * 64 + half * 32 + (s % 2) * 16 + j
+    return out_col + (s >= 2) * F
+
+
+def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit: float, slope: float, shift: float, act_dtype, tiled: bool = False):
+    """``tiled``: every expert's rows of w_gu are in :func:`moe_glu_row_order` (bfloat16 on the GPU, d and F on the
+    128 grid): prompt-sized batches then run as grouped matrix-core GEMMs."""
     if _gpu(h):
-        return _k().hy_moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift)
+        return _k().hy_moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, tiled)
+    if tiled:
+        w_gu = w_gu[:, torch.argsort(moe_glu_row_order(w_gu.shape[1] // 2)).to(w_gu.device)]
     return ref.moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, act_dtype)

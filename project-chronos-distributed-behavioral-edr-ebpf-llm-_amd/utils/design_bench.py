@@ -1,8 +1,10 @@
-"""Throughput of a hybrid design (Zokunex) beside the Llama family at equal width and depth: whole-model prefill and
-decode steps, and each new kernel beside its closest Llama kernel with the fraction of its roofline it reaches.
+"""Throughput of a hybrid design (Zokunex, Kalesun) beside the framework's other models at equal width and depth:
+whole-model prefill and decode steps, and each of the design's kernels beside its closest existing kernel with the
+fraction of its roofline it reaches.
 
-``python bench.py --design-compare [--design-sizes 1k,2k,4k]`` prints one JSON line (the default benchmark and its
-output line are untouched).  Weights are random; every number is measured on the GPU this process runs on.
+``python bench.py --design-compare [--design zokunex|kalesun] [--design-sizes 1k,2k,4k]`` prints one JSON line (the
+default benchmark and its output line are untouched).  Zokunex stands beside Llama; Kalesun beside Zokunex (the
+closest family: recurrent layers, attention and mixtures of experts on a float32 stream) and Llama.  Weights are random; every number is measured on the GPU this process runs on.
 
 Rooflines: HBM 8 TB/s for kernels bound by the bytes they must move, 2.5 PFLOP/s dense bf16 for the matrix-shaped
 ones (the attention kernels over a long context are priced by their FLOPs in prefill and by their cache bytes in
@@ -40,6 +42,33 @@ def zokunex_config(size: dict) -> dict:
     moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=ne, identity=ni, top=top))
     layers = [dict(mix_m, mlp=dense), dict(mix_a, mlp=moe), dict(mix_m, mlp=moe), dict(mix_a, mlp=dense)][:LAYERS]
     return dict(architecture="Zokunex", vocab=VOCAB, width=size["width"], logit_scale=1.0, norm=dict(eps=1e-5),
+                layers=layers)
+
+
+# Kalesun: width -> (attention heads, kv heads, dim, vdim, window, kept | delta heads, qk heads, dim, vdim |
+#                    gla heads, dim, vdim | dense ff | experts, top, expert ff)
+KALESUN_SIZES = {
+    "1k": dict(width=1024, a=(8, 2, 128, 128, 512, 4), d=(8, 4, 128, 128), g=(4, 128, 256), ff=2816, moe=(8, 2, 512)),
+    "2k": dict(width=2048, a=(16, 4, 128, 128, 1024, 4), d=(16, 8, 128, 128), g=(8, 128, 256), ff=5632, moe=(16, 4, 1024)),
+    "4k": dict(width=4096, a=(32, 8, 128, 128, 1024, 4), d=(32, 16, 128, 128), g=(16, 128, 256), ff=11008, moe=(32, 4, 1536)),
+}
+
+
+def kalesun_config(size: dict) -> dict:
+    ah, ag, ad, av, win, keep = size["a"]
+    dh, dk, dd, dv = size["d"]
+    gh, gd, gv = size["g"]
+    ne, top, eff = size["moe"]
+    mix_a = dict(type="attention", mixer=dict(heads=ah, kv_heads=ag, dim=ad, vdim=av, scale=ad ** -0.5, v_mix=True,
+                                              mask=dict(size=win, keep_first=keep),
+                                              rot=dict(base=500000.0, dims=ad // 2,
+                                                       scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192))))
+    mix_d = dict(type="delta", mixer=dict(heads=dh, kv_heads=dk, dim=dd, vdim=dv, conv=4))
+    mix_g = dict(type="gla", mixer=dict(heads=gh, dim=gd, vdim=gv, tau=16.0, rank=16))
+    dense = dict(kind="dense", ff=size["ff"], limit=7.0)
+    moe = dict(kind="moe", expert=dict(ff=eff, limit=7.0), router=dict(experts=ne, top=top))
+    layers = [dict(mix_d, mlp=dense), dict(mix_a, mlp=moe), dict(mix_g, mlp=moe), dict(mix_a, mlp=dense)][:LAYERS]
+    return dict(architecture="Kalesun", vocab=VOCAB, width=size["width"], postln_alpha=2.0, norm=dict(eps=1e-6),
                 layers=layers)
 
 
@@ -190,6 +219,190 @@ def _kernels(size: dict, dev, T: int, ctx: int, rows: int) -> dict:
     return out
 
 
+def _kernels_kalesun(size: dict, zsize: dict, dev, T: int, ctx: int, rows: int) -> dict:
+    """Kalesun's kernels and their closest existing kernels at this size: seconds, and the fraction of the roofline
+    reached.  ``zsize``: the Zokunex sizes of the same width (for the kernels it stands beside)."""
+    from chronos import ops
+    from chronos.models.hybrid import rope_cos_sin
+    from chronos.ops import hybrid as hops
+
+    out = {}
+    bf = torch.bfloat16
+    d = size["width"]
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *s, dt=bf, sc=1.0: (torch.randn(*s, device=dev, generator=g) * sc).to(dt)  # noqa: E731
+    i32 = dict(dtype=torch.int32, device=dev)
+
+    def rec(name, secs, nbytes=0.0, flops=0.0):
+        roof = max(nbytes / HBM_BPS, flops / BF16_FLOPS)
+        _say(f"  {name}: {secs * 1e6:.1f} us, roofline {roof * 1e6:.2f} us")
+        out[name] = dict(us=round(secs * 1e6, 1), roofline_us=round(roof * 1e6, 2), of_roofline=round(roof / secs, 4))
+
+    # ---- norms on the residual stream
+    y, x32, w32 = rnd(T, d), rnd(T, d, dt=torch.float32), rnd(d, dt=torch.float32)
+    rec("scale_add_rms_norm", _time(lambda: hops.scale_add_rms_norm(y, x32, w32, 2.0, 1e-6, bf)), T * d * (2 + 4 + 4 + 2))
+    rec("zokunex.add_layer_norm", _time(lambda: hops.add_layer_norm(y, x32, w32, 1e-5, bf)), T * d * (2 + 4 + 4 + 2))
+    xb, wb = rnd(T, d), rnd(d)
+    rec("llama.add_rmsnorm", _time(lambda: ops.add_rmsnorm(y, xb, wb, 1e-5)), T * d * (2 + 2 + 2 + 2))
+    # ---- attention: prefill of T tokens (seqs of `ctx`), decode of `rows` rows at context ctx
+    H, G, D, Dv, win, keep = size["a"]
+    bs = 16
+    seqs = max(1, T // ctx)
+    per = ctx // bs + 1
+    nb = max(seqs, rows) * per + 1
+    kc, vc = rnd(nb, bs, G, D, sc=0.3), rnd(nb, bs, G, Dv, sc=0.3)
+    C = (H + G) * D + G * Dv
+    qkv = rnd(seqs * ctx, C, sc=0.3)
+    gate, sink = rnd(seqs * ctx, H, dt=torch.float32), rnd(H, dt=torch.float32)
+    bt = torch.arange(1, 1 + seqs * per, **i32).view(seqs, per)
+    qs = torch.arange(0, (seqs + 1) * ctx, ctx, **i32)
+    pos = torch.arange(ctx, **i32).repeat(seqs)
+    tseq = torch.arange(seqs, **i32).repeat_interleave(ctx)
+    vis = sum(min(i + 1, win) + max(0, min(keep, i + 1 - win)) for i in range(ctx))  # visible (query, key) pairs
+    pairs = seqs * vis
+    rec("window_attention.prefill", _time(lambda: hops.window_attention(qkv, kc, vc, bt, qs, pos, sink, gate, D ** -0.5, win, keep, H, bf, ctx), iters=3, warm=1),
+        flops=2.0 * pairs * H * (D + Dv))
+    cs = rope_cos_sin(500000.0, D // 2, ctx + 1, dev, (8.0, 1.0, 4.0, 8192.0))
+    qn, vf, lam = rnd(D, dt=torch.float32), rnd(seqs * ctx, G * Dv), torch.tensor([0.3], device=dev)
+    rec("window_prep.prefill", _time(lambda: hops.window_prep(qkv, H, G, D, Dv, vf, lam, pos, tseq, bt, qn, qn, 1e-6, cs, D // 2, kc, vc, False)),
+        nbytes=seqs * ctx * (C * 2 + H * D * 2 + 2 * G * (D + Dv) * 2.0))
+    btd = torch.arange(1, 1 + rows * per, **i32).view(rows, per)
+    qsd = torch.arange(rows + 1, **i32)
+    posd = torch.full((rows,), ctx, **i32)
+    qkvd, gated = rnd(rows, C, sc=0.3), rnd(rows, H, dt=torch.float32)
+    rec("window_attention.decode", _time(lambda: hops.window_attention(qkvd, kc, vc, btd, qsd, posd, sink, gated, D ** -0.5, win, keep, H, bf, 1)),
+        nbytes=rows * (min(ctx + 1, win) + keep) * G * (D + Dv) * 2.0)
+    # beside: Llama's paged GQA attention (full causal) and Zokunex's latent attention at this width
+    hq = d // 128
+    hkv = max(1, hq // 4)
+    lkc, lvc = rnd(nb, hkv, bs, 128, sc=0.3), rnd(nb, hkv, 128, bs, sc=0.3)
+    q = rnd(seqs * ctx, hq, 128, sc=0.3)
+    ctxl = torch.full((seqs,), ctx, **i32)
+    tiles = torch.tensor(ops.attention_tiles([ctx] * seqs, hq, hkv, 8), **i32).view(-1, 2)
+    full_pairs = seqs * ctx * (ctx + 1) / 2
+    rec("llama.attention.prefill", _time(lambda: ops.paged_attention(q, lkc, lvc, bt, qs, ctxl, tiles, tiles.shape[0], 8, 1), iters=3, warm=1),
+        flops=4.0 * full_pairs * hq * 128)
+    qd = rnd(rows, hq, 128, sc=0.3)
+    ctxd = torch.full((rows,), ctx + 1, **i32)
+    ns = ops.pick_nsplit(rows * hkv, ctx + 1)
+    rec("llama.attention.decode", _time(lambda: ops.paged_attention(qd, lkc, lvc, btd, qsd, ctxd, None, rows, 1, ns)),
+        nbytes=rows * (ctx + 1) * hkv * 128 * 2 * 2.0)
+    zh, zd, zr, zv, rank = zsize["a"]
+    DK = rank + zr
+    lat = rnd(nb, bs, DK, sc=0.3)
+    qa, zg = rnd(seqs * ctx, zh, DK, sc=0.3), rnd(seqs * ctx, zh, dt=torch.float32)
+    rec("zokunex.latent_attention.prefill", _time(lambda: hops.latent_attention(qa, lat, bt, qs, pos, zg, 0.1, rank, bf, ctx), iters=3, warm=1),
+        flops=2.0 * full_pairs * zh * (DK + rank))
+    qad, zgd = rnd(rows, zh, DK, sc=0.3), rnd(rows, zh, dt=torch.float32)
+    rec("zokunex.latent_attention.decode", _time(lambda: hops.latent_attention(qad, lat, btd, qsd, posd, zgd, 0.1, rank, bf, 1)),
+        nbytes=rows * (ctx + 1) * DK * 2.0)
+    # ---- the recurrences: prefill (FLOPs of the state update and read-out), decode (state bytes in and out)
+    NS = max(seqs, rows) + 1
+    p0, sl, sld = torch.zeros(seqs, **i32), torch.arange(seqs, **i32), torch.arange(rows, **i32)
+    for name, (hh, hk, dd, dv), delta in (("delta", size["d"], True), ("gla", (size["g"][0], size["g"][0], *size["g"][1:]), False)):
+        Cq = 2 * hk * dd + hh * dv
+        S = torch.zeros(NS, hh, dd, dv, device=dev)
+
+        def scan(proj, qs_, p0_, sl_, n):
+            if delta:
+                qsc, ksc = torch.rand(n, hk, device=dev), torch.rand(n, hk, device=dev)
+                dec, beta = torch.rand(n, hh, device=dev), torch.rand(n, hh, device=dev)
+                return lambda: hops.linear_scan(proj, 0, hk * dd, 2 * hk * dd, qsc, ksc, 1.0, dec, beta, qs_, p0_, sl_, S, hk, hh, dd, dv)
+            dec = torch.rand(n, hh, dd, device=dev)
+            return lambda: hops.linear_scan(proj, 0, hk * dd, 2 * hk * dd, None, None, dd ** -0.5, dec, None, qs_, p0_, sl_, S, hk, hh, dd, dv)
+
+        proj = rnd(seqs * ctx, Cq, sc=0.5)
+        rec(f"linear_scan.{name}.prefill", _time(scan(proj, qs, p0, sl, seqs * ctx), iters=3, warm=1),
+            nbytes=seqs * ctx * Cq * 2.0, flops=seqs * ctx * hh * dd * dv * (6.0 if delta else 4.0))
+        projd = rnd(rows, Cq, sc=0.5)
+        rec(f"linear_scan.{name}.decode", _time(scan(projd, qsd, posd, sld, rows)), nbytes=rows * hh * dd * dv * 4 * 2.0)
+    dh, dk, dd, dv = size["d"]
+    Cc = 2 * dk * dd + dh * dv
+    xc, taps = rnd(seqs * ctx, Cc + dh * dv), rnd(Cc, 4, dt=torch.float32)
+    hist = torch.zeros(NS, 3, Cc, device=dev, dtype=bf)
+    rec("short_conv.prefill", _time(lambda: hops.short_conv(xc, taps, tseq, qs, p0, sl, hist, True)), nbytes=seqs * ctx * Cc * 4.0)
+    mh, md, mv = zsize["m"]
+    Cm = 2 * mh * md + 2 * mh * mv
+    mproj, gp = rnd(seqs * ctx, Cm, sc=0.5), rnd(seqs * ctx, 2 * mh, dt=torch.float32)
+    mS, mn, mm = (torch.zeros(NS, mh, md, mv, device=dev), torch.zeros(NS, mh, md, device=dev), torch.zeros(NS, mh, device=dev))
+    rec("zokunex.mlstm_scan.prefill", _time(lambda: hops.mlstm_scan(mproj, gp, qs, p0, sl, mS, mn, mm, mh, md, mv, 10.0, ctx), iters=3, warm=1),
+        nbytes=seqs * ctx * Cm * 2.0, flops=seqs * ctx * mh * md * mv * 6.0)
+    mprojd, gpd = rnd(rows, Cm, sc=0.5), rnd(rows, 2 * mh, dt=torch.float32)
+    rec("zokunex.mlstm_scan.decode", _time(lambda: hops.mlstm_scan(mprojd, gpd, qsd, posd, sld, mS, mn, mm, mh, md, mv, 10.0, 1)),
+        nbytes=rows * mh * md * mv * 4 * 2.0)
+    # ---- feed-forwards: gated experts beside Zokunex's experts and Llama's dense SwiGLU; the gated unit's activation
+    ne, top, eff = size["moe"]
+    wr, br = rnd(ne, d, sc=0.05), rnd(ne, dt=torch.float32, sc=0.01)
+    wgu = rnd(ne, 2 * eff, d, sc=d ** -0.5)[:, hops.moe_glu_row_order(eff).to(dev)].contiguous()
+    wd = rnd(ne, d, eff, sc=eff ** -0.5)
+    ze, zi, ztop, zeff = zsize["moe"]
+    zwr, zcorr = rnd(ze + zi, d, sc=0.05), rnd(ze + zi, dt=torch.float32, sc=0.01)
+    zwu, zwd = rnd(ze, zeff, d, sc=d ** -0.5), rnd(ze, d, zeff, sc=zeff ** -0.5)
+    for name, tk in (("prefill", T), ("decode", rows)):
+        h = rnd(tk, d)
+        idx, wt = hops.moe_route_topk(h, wr, br, top)
+        rec(f"moe_route_topk.{name}", _time(lambda: hops.moe_route_topk(h, wr, br, top)), nbytes=tk * d * 2.0 + ne * d * 2.0)
+        used = min(ne, tk * top) * 3 * eff * d * 2.0
+        rec(f"moe_glu_ffn.{name}", _time(lambda: hops.moe_glu_ffn(h, idx, wt, wgu, wd, 7.0, 1.702, 1.0, bf, True), iters=3, warm=1),
+            nbytes=used + tk * d * 4.0, flops=tk * top * 6.0 * eff * d)
+        zidx, zwt = hops.moe_route(h, zwr, zcorr, ztop)
+        real = float((zidx < ze).sum())
+        rec(f"zokunex.moe_ffn.{name}", _time(lambda: hops.moe_ffn(h, zidx, zwt, zwu, zwd, 1, bf), iters=3, warm=1),
+            nbytes=min(ze, real) * 2 * zeff * d * 2.0 + tk * d * 4.0, flops=real * 4.0 * zeff * d)
+        f = size["ff"]
+        gu = rnd(tk, 2 * f)
+        rec(f"glu.{name}", _time(lambda: hops.glu(gu, 7.0, 1.702, 1.0, bf)), nbytes=tk * f * 6.0)
+        lf = int(3.5 * d)
+        wgl, wdn = rnd(2 * lf, d, sc=d ** -0.5), rnd(d, lf, sc=lf ** -0.5)
+        rec(f"llama.mlp.{name}", _time(lambda: ops.linear(ops.gate_up_silu(h, wgl), wdn), iters=3, warm=1),
+            nbytes=3 * lf * d * 2.0 + tk * d * 4.0, flops=tk * 6.0 * lf * d)
+    return out
+
+
+def run_kalesun(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
+    from chronos import ops
+    from chronos.models import kalesun, llama, zokunex
+    from chronos.models.hybrid import HybridDecoder
+
+    dev = torch.device(device if ":" in device else device + ":0")
+    torch.cuda.set_device(dev)
+    ops.load()
+    ops.device_init()
+    res = {}
+    P = ctx + plen + 16
+    for name in sizes:
+        size, zsize = KALESUN_SIZES[name], SIZES[name]
+        t0 = time.time()
+        cfg = kalesun.config_from_dict(kalesun_config(size), name=f"kalesun-{name}", max_position=P)
+        km = HybridDecoder(cfg, kalesun.pack_weights(cfg, kalesun.random_tensors(cfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry = dict(kalesun=dict(params=cfg.param_count(), **_model_steps(km, dev, seqs, plen, rows, ctx)))
+        _say(f"size {name}: kalesun {entry['kalesun']}")
+        del km
+        zcfg = zokunex.config_from_dict(zokunex_config(zsize), name=f"zokunex-{name}", max_position=P)
+        zk = HybridDecoder(zcfg, zokunex.pack_weights(zcfg, zokunex.random_tensors(zcfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry["zokunex"] = dict(params=zcfg.param_count(), **_model_steps(zk, dev, seqs, plen, rows, ctx))
+        _say(f"  zokunex {entry['zokunex']}")
+        del zk
+        d = size["width"]
+        lc = llama.LlamaConfig(name=f"llama-{name}", vocab_size=VOCAB, hidden_size=d, intermediate_size=int(3.5 * d),
+                               num_layers=LAYERS, num_heads=d // 128, num_kv_heads=max(1, d // 512), max_position=P)
+        lm = llama.LlamaModel(lc, llama.random_weights(lc, None, dev, 0), None, dev, P)
+        entry["llama"] = dict(params=lc.param_count(), **_model_steps(lm, dev, seqs, plen, rows, ctx))
+        _say(f"  llama {entry['llama']}")
+        del lm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _kernels_kalesun(size, zsize, dev, seqs * plen, ctx, rows)
+        entry["seconds"] = round(time.time() - t0, 1)
+        res[name] = entry
+        torch.cuda.empty_cache()
+    return dict(metric="design_compare", design="kalesun", beside="zokunex and llama (equal width and depth)",
+                layers=LAYERS, workload=dict(prefill=f"{seqs} x {plen} tokens in one step",
+                                             decode=f"{rows} rows at context {ctx}"),
+                dtype="bf16", data="synthetic", sizes=res)
+
+
 def run(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
     from chronos import ops
     from chronos.models import llama, zokunex
@@ -227,6 +440,7 @@ def run(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int =
 
 
 def main(a) -> int:
-    out = run([s for s in a.design_sizes.split(",") if s], device=a.device)
+    sizes = [s for s in a.design_sizes.split(",") if s]
+    out = (run_kalesun if getattr(a, "design", "zokunex") == "kalesun" else run)(sizes, device=a.device)
     print(json.dumps(out), flush=True)
     return 0

@@ -91,7 +91,9 @@ def _stream(lens, starts, bs, nblocks, gen):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("H,G,D,Dv,dims,window,keep", [(4, 2, 24, 40, 8, 9, 3), (3, 3, 64, 16, 64, 0, 0),
-                                                       (6, 1, 16, 72, 0, 70, 5), (2, 2, 128, 128, 32, 130, 66)])
+                                                       (6, 1, 16, 72, 0, 70, 5), (2, 2, 128, 128, 32, 130, 66),
+                                                       (6, 2, 64, 48, 16, 20, 70), (12, 1, 32, 16, 32, 0, 0),
+                                                       (4, 4, 256, 256, 64, 64, 1), (5, 1, 96, 80, 0, 3, 0)])
 def test_window_attention(dt, H, G, D, Dv, dims, window, keep):
     from chronos.models.hybrid import rope_cos_sin
     from chronos.ops import hybrid as hops, hybrid_ref as ref
@@ -210,6 +212,24 @@ def test_moe_glu(dt, T, d, F, E, top):
     wd = _rand(g, E, d, F, dtype=dt, scale=F ** -0.5)
     _close(hops.moe_glu_ffn(h, idx, wt, wgu, wd, 1.5, 1.702, 1.0, dt),
            ref.moe_glu_ffn(h, idx2, wt2, wgu, wd, 1.5, 1.702, 1.0, dt), _tol(dt, 2e-5, 1.5e-2))
+
+
+@pytest.mark.parametrize("T,d,F,E,top", [(200, 256, 128, 4, 2), (90, 128, 384, 3, 3)])
+def test_moe_glu_tile_order(T, d, F, E, top):
+    """bfloat16 experts in the grouped path's row order: prompt-sized batches on the grouped matrix-core GEMMs and a
+    few rows on the token kernel, both against the reference on the natural row order."""
+    from chronos.ops import hybrid as hops, hybrid_ref as ref
+
+    dt = torch.bfloat16
+    g = _gen(T + F)
+    h = _rand(g, T, d, dtype=dt)
+    idx, wt = hops.moe_route_topk(h, _rand(g, E, d, dtype=dt, scale=0.5), _rand(g, E), top)
+    wgu = _rand(g, E, 2 * F, d, dtype=dt, scale=d ** -0.5)
+    wd = _rand(g, E, d, F, dtype=dt, scale=F ** -0.5)
+    tiled = wgu[:, hops.moe_glu_row_order(F).to(DEV)].contiguous()
+    want = ref.moe_glu_ffn(h, idx, wt, wgu, wd, 2.0, 1.702, 1.0, dt)
+    _close(hops.moe_glu_ffn(h, idx, wt, tiled, wd, 2.0, 1.702, 1.0, dt, True), want, 1.5e-2)
+    _close(hops.moe_glu_ffn(h[:3], idx[:3], wt[:3], tiled, wd, 2.0, 1.702, 1.0, dt, True), want[:3], 1.5e-2)
 
 
 def test_router_ties_go_to_the_lower_index():
