@@ -128,7 +128,7 @@ def test_window_attention(dt, H, G, D, Dv, dims, window, keep):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("C,K", [(70, 4), (300, 2), (17, 1), (64, 7)])
+@pytest.mark.parametrize("C,K", [(70, 4), (300, 2), (17, 1), (64, 7), (1024 + 16, 4), (8, 3)])
 def test_short_conv(dt, C, K):
     from chronos.ops import hybrid as hops, hybrid_ref as ref
 
@@ -136,7 +136,7 @@ def test_short_conv(dt, C, K):
     lens, starts, slots = [5, 1, 1, 9, 2], [0, 4, 0, 7, 3], [2, 0, 4, 1, 3]
     pos, seq, bt, qs = _stream(lens, starts, 16, 16, g)
     T = int(qs[-1])
-    x = _rand(g, T, C + 13, dtype=dt)
+    x = _rand(g, T, C + (13 if C % 8 else 24), dtype=dt)
     w = _rand(g, C, K, scale=0.5)
     hist = _rand(g, 6, K - 1, C, dtype=dt)
     hist2 = hist.clone()
