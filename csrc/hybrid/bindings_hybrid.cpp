@@ -47,7 +47,8 @@ void launch_hy_window_prep(void*, int, int, int, int, int, const void*, const fl
 int hy_window_rows_cap(int, int, int, bool);
 void launch_hy_window_attention(const void*, int, const void*, const void*, const int32_t*, int, const int32_t*,
                                 const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
-                                int, int, bool, hipStream_t);
+                                int, int, bool, int, float*, float*, int64_t, hipStream_t);
+int hy_window_nsplit(bool, int, int, int, int, int, int, int, int, int, int);
 void launch_hy_short_conv(const void*, int, const float*, const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                           void*, void*, int, int, int, int, bool, bool, hipStream_t);
 void launch_hy_delta_prep(const void*, int, const float*, const float*, float*, float*, float*, float*, int, int, int, int,
@@ -393,12 +394,22 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
     if (gate) { flt(*gate, "window_attention: float32 gate"); need(gate->numel() == T * H, "window_attention: gate [T, H]"); }
     auto out = at::empty({T, H * Dv}, qkv.options());
     if (T == 0 || B <= 0) return out;
+    const int mq = (int)std::max<int64_t>(1, max_q);
+    const int nsplit = chronos::hy_window_nsplit(f32(qkv), (int)qkv.size(1), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv,
+                                                 (int)window, (int)keep, (int)(block_table.size(1) * kc.size(1)));
+    Tensor part_o, part_ml;
+    if (nsplit > 1) {
+        part_o = at::empty({T * H * nsplit, Dv}, qkv.options().dtype(at::kFloat));
+        part_ml = at::empty({T * H * nsplit, 2}, qkv.options().dtype(at::kFloat));
+    }
     chronos::launch_hy_window_attention(qkv.data_ptr(), (int)qkv.size(1), kc.data_ptr(), vc.data_ptr(),
                                         block_table.data_ptr<int32_t>(), (int)block_table.size(1),
                                         q_start.data_ptr<int32_t>(), pos.data_ptr<int32_t>(),
                                         sink ? sink->data_ptr<float>() : nullptr, gate ? gate->data_ptr<float>() : nullptr,
-                                        out.data_ptr(), (int)B, (int)std::max<int64_t>(1, max_q), (int)H, (int)G, (int)D,
-                                        (int)Dv, (int)kc.size(1), (float)scale, (int)window, (int)keep, f32(qkv), stream());
+                                        out.data_ptr(), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv, (int)kc.size(1),
+                                        (float)scale, (int)window, (int)keep, f32(qkv), nsplit,
+                                        nsplit > 1 ? part_o.data_ptr<float>() : nullptr,
+                                        nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, T * H, stream());
     return out;
 }
 

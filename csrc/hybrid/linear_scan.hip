@@ -20,28 +20,7 @@
 namespace chronos {
 namespace hy {
 
-template <typename T> struct ConvVec { static constexpr int E = 16 / (int)sizeof(T); };
-template <typename T> __device__ __forceinline__ void unpack_row16(const T* p, float* f);
-template <> __device__ __forceinline__ void unpack_row16<uint16_t>(const uint16_t* p, float* f) {
-    const u16x8 v = *reinterpret_cast<const u16x8*>(p);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = bf2f(v[i]);
-}
-template <> __device__ __forceinline__ void unpack_row16<float>(const float* p, float* f) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = v[i];
-}
-template <typename T> __device__ __forceinline__ void pack_row16(T* p, const float* f);
-template <> __device__ __forceinline__ void pack_row16<uint16_t>(uint16_t* p, const float* f) {
-    *reinterpret_cast<u16x8*>(p) = u16x8{f2bf(f[0]), f2bf(f[1]), f2bf(f[2]), f2bf(f[3]), f2bf(f[4]), f2bf(f[5]), f2bf(f[6]), f2bf(f[7])};
-}
-template <> __device__ __forceinline__ void pack_row16<float>(float* p, const float* f) {
-    *reinterpret_cast<f32x4*>(p) = f32x4{f[0], f[1], f[2], f[3]};
-}
-
-// VEC: a thread takes 16 bytes of consecutive channels (C, ldx and the row starts on 16-byte boundaries).
-template <typename T, bool VEC>
+template <typename T>
 __global__ void __launch_bounds__(256) short_conv_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
                                                          const int32_t* __restrict__ tok_seq,
                                                          const int32_t* __restrict__ q_start,
@@ -53,40 +32,17 @@ __global__ void __launch_bounds__(256) short_conv_kernel(const T* __restrict__ x
     const int t0 = q_start[b];
     const bool past = pos0[b] > 0;
     const T* hrow = hist + (int64_t)slots[b] * (K - 1) * C;
-    if constexpr (VEC) {
-        constexpr int E = ConvVec<T>::E;
-        for (int c = (blockIdx.y * 256 + threadIdx.x) * E; c < C; c += gridDim.y * 256 * E) {
-            float acc[E];
-#pragma unroll
-            for (int e = 0; e < E; ++e) acc[e] = 0.f;
-            for (int i = 0; i < K; ++i) {
-                const int64_t s = t - (K - 1) + i;
-                float v[E];
-                if (s >= t0) unpack_row16<T>(x + s * ldx + c, v);
-                else if (past) unpack_row16<T>(hrow + (int64_t)((K - 1) + (s - t0)) * C + c, v);
-                else continue;
-#pragma unroll
-                for (int e = 0; e < E; ++e) acc[e] += w[(c + e) * K + i] * v[e];
-            }
-            if (silu) {
-#pragma unroll
-                for (int e = 0; e < E; ++e) acc[e] = acc[e] * sigmoidf_(acc[e]);
-            }
-            pack_row16<T>(y + t * C + c, acc);
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float acc = 0.f;
+        for (int i = 0; i < K; ++i) {
+            const int64_t s = t - (K - 1) + i;
+            float v = 0.f;
+            if (s >= t0) v = ld<T>(x + s * ldx + c);
+            else if (past) v = ld<T>(hrow + (int64_t)((K - 1) + (s - t0)) * C + c);
+            acc += w[c * K + i] * v;
         }
-    } else {
-        for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
-            float acc = 0.f;
-            for (int i = 0; i < K; ++i) {
-                const int64_t s = t - (K - 1) + i;
-                float v = 0.f;
-                if (s >= t0) v = ld<T>(x + s * ldx + c);
-                else if (past) v = ld<T>(hrow + (int64_t)((K - 1) + (s - t0)) * C + c);
-                acc += w[c * K + i] * v;
-            }
-            if (silu) acc = acc * sigmoidf_(acc);
-            st<T>(y + t * C + c, acc);
-        }
+        if (silu) acc = acc * sigmoidf_(acc);
+        st<T>(y + t * C + c, acc);
     }
 }
 
@@ -297,18 +253,10 @@ void launch_hy_short_conv(const void* x, int ldx, const float* w, const int32_t*
     if (T == 0 || C == 0) return;
     const dim3 hg(B, (C + 255) / 256);
     if (f32) {
-        constexpr int E = hy::ConvVec<float>::E;
-        if (C % E == 0 && ldx % E == 0)
-            hy::short_conv_kernel<float, true><<<dim3(T, (C / E + 255) / 256), 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu);
-        else
-            hy::short_conv_kernel<float, false><<<dim3(T, (C + 255) / 256), 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu);
+        hy::short_conv_kernel<float><<<T, 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu);
         if (K > 1) hy::conv_hist_kernel<float><<<hg, 256, 0, s>>>((const float*)x, ldx, q_start, pos0, slots, (float*)hist, C, K);
     } else {
-        constexpr int E = hy::ConvVec<uint16_t>::E;
-        if (C % E == 0 && ldx % E == 0)
-            hy::short_conv_kernel<uint16_t, true><<<dim3(T, (C / E + 255) / 256), 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu);
-        else
-            hy::short_conv_kernel<uint16_t, false><<<dim3(T, (C + 255) / 256), 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu);
+        hy::short_conv_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu);
         if (K > 1) hy::conv_hist_kernel<uint16_t><<<hg, 256, 0, s>>>((const uint16_t*)x, ldx, q_start, pos0, slots, (uint16_t*)hist, C, K);
     }
 }

@@ -250,17 +250,19 @@ int hy_window_rows_cap(int R, int D, int Dv, bool f32) {
 
 bool launch_hy_window_attention_mfma(const uint16_t*, int, const uint16_t*, const uint16_t*, const int32_t*, int,
                                      const int32_t*, const int32_t*, const float*, const float*, uint16_t*, int, int, int,
-                                     int, int, int, int, float, int, int, hipStream_t);
+                                     int, int, int, int, float, int, int, int, float*, float*, int64_t, hipStream_t);
 
 // bfloat16 at matrix-core sizes runs window_attention_mfma.hip; float32 and every other size the general kernel.
 void launch_hy_window_attention(const void* qkv, int ld, const void* kc, const void* vc, const int32_t* block_table,
                                 int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
                                 const float* gate, void* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
-                                float scale, int window, int keep, bool f32, hipStream_t s) {
+                                float scale, int window, int keep, bool f32, int nsplit, float* part_o, float* part_ml,
+                                int64_t total_rows, hipStream_t s) {
     if (B == 0 || max_q == 0) return;
     if (!f32 && launch_hy_window_attention_mfma((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc,
                                                 block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, B,
-                                                max_q, H, G, D, Dv, BS, scale, window, keep, s))
+                                                max_q, H, G, D, Dv, BS, scale, window, keep, nsplit, part_o, part_ml,
+                                                total_rows, s))
         return;
     const int R = H / G;   // the caller has checked R <= 64, Dv <= 256 and that hy_window_rows_cap is not 0
     const int rows_cap = hy_window_rows_cap(R, D, Dv, f32);

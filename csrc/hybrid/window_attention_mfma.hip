@@ -15,8 +15,11 @@
 //   * sum  O^T = V^T P^T : the lane's 8 weights of two neighbouring 16-key tiles ARE a B operand (the k index is a
 //     fixed permutation of the 32 keys, the same one the transposed value image is read with); each weight enters
 //     as two bfloat16 terms (rounded value + remainder), which keeps the float softmax weights nearly exact.
-// After the last tile the head's sink joins the denominator and the row is scaled by sigmoid(gate).
+// After the last tile the head's sink joins the denominator and the row is scaled by sigmoid(gate).  Launches of few
+// rows (decode) deal a row block's key tiles to several workgroups and merge the float partials in a second kernel.
 // Sizes: D % 32 == 0, Dv % 16 == 0, D <= 256, Dv <= 256.  Everything else takes the general kernel.
+#include <algorithm>
+
 #include "hybrid_common.h"
 
 namespace chronos {
@@ -29,14 +32,16 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
         const uint16_t* __restrict__ qkv, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
         const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
         const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
-        uint16_t* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep) {
+        uint16_t* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int nsplit,
+        float* __restrict__ part_o, float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int KT = WKT, NT = 64 * NW, RPB = 16 * NW, PP = KT / 2;
     const int R = H / G;
     const int b = blockIdx.x, kvh = blockIdx.z;
     const int t0 = q_start[b], t1 = q_start[b + 1];
     const int rows_total = (t1 - t0) * R;
-    const int rb0 = blockIdx.y * RPB;
+    const int split = blockIdx.y % nsplit;   // key tiles are dealt round-robin to the nsplit workgroups of a row block
+    const int rb0 = blockIdx.y / nsplit * RPB;
     if (rb0 >= rows_total) return;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, g4 = lane >> 4, qi = lane & 15;
     const int ns = D / 32, nct = Dv / 16;
@@ -61,6 +66,7 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
 #pragma unroll
     for (int c = 0; c < NCT; ++c) O[c] = f32x4{0.f, 0.f, 0.f, 0.f};
     float mrow = -INFINITY, lrow = 0.f;
+    const float scale2 = scale * 1.4426950408889634f;
     const int32_t* bt = block_table + (int64_t)b * max_blocks;
     const int kchunks = D / 8, vchunks = Dv / 8;
     const int w_lo = window > 0 ? max(0, pmin - window + 1) : 0;
@@ -70,7 +76,7 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
     const int k_end = window > 0 ? min(keep, w_start) : 0;
     const int n_keep_tiles = (k_end + KT - 1) / KT;
     const int n_tiles = n_keep_tiles + (pmax - w_start) / KT + 1;
-    for (int ti = 0; ti < n_tiles; ++ti) {
+    for (int ti = split; ti < n_tiles; ti += nsplit) {
         const bool kept = ti < n_keep_tiles;
         const int k0 = kept ? ti * KT : w_start + (ti - n_keep_tiles) * KT;
         const int k_last = kept ? k_end - 1 : pmax;  // last real key this tile may hold
@@ -110,27 +116,42 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
                     S[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(arow + s * 64), qf[s],
                                                                     S[kt], 0, 0, 0);
         }
+        // scores, maxima and sums live in the base-2 domain (score * scale * log2 e): one multiply and one
+        // subtraction in front of the hardware's exp2.  A tile that every row of the block sees whole (the common case
+        // inside a window) skips the per-key visibility tests.
+        const bool whole = k0 + KT - 1 <= min(k_last, pmin) && (window <= 0 || kept || pmax - k0 < window);
         float mx = -INFINITY;
+        if (whole) {
 #pragma unroll
-        for (int kt = 0; kt < NKT; ++kt)
+            for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = k0 + 16 * kt + 4 * g4 + i;
-                const bool vis = key <= k_last && key <= prow && (window <= 0 || prow - key < window || key < keep);
-                const float sv = vis ? S[kt][i] * scale : -INFINITY;
-                S[kt][i] = sv;
-                mx = fmaxf(mx, sv);
-            }
+                for (int i = 0; i < 4; ++i) {
+                    S[kt][i] *= scale2;
+                    mx = fmaxf(mx, S[kt][i]);
+                }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = k0 + 16 * kt + 4 * g4 + i;
+                    const bool vis = key <= k_last && key <= prow && (window <= 0 || prow - key < window || key < keep);
+                    const float sv = vis ? S[kt][i] * scale2 : -INFINITY;
+                    S[kt][i] = sv;
+                    mx = fmaxf(mx, sv);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(mrow, mx);
-        const float corr = (mn == -INFINITY) ? 1.f : __expf(mrow - mn);
+        const float corr = (mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mrow - mn);
+        const float mref = (mn == -INFINITY) ? 0.f : mn;  // (all masked: every exponent is -inf, every weight 0)
         float sum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = (mn == -INFINITY) ? 0.f : __expf(S[kt][i] - mn);
+                const float p = __builtin_amdgcn_exp2f(S[kt][i] - mref);
                 S[kt][i] = p;
                 sum += p;
             }
@@ -170,12 +191,23 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
         }
     }
     if (!rok) return;
+    if (nsplit > 1) {  // unnormalised partial: the combine kernel merges the splits and adds sink and gate
+        const int64_t pr = (tok * H + head) * nsplit + split;
+        if (g4 == 0) {
+            part_ml[pr * 2] = mrow;
+            part_ml[pr * 2 + 1] = lrow;
+        }
+#pragma unroll
+        for (int c = 0; c < NCT; ++c)
+            if (c < nct) *reinterpret_cast<f32x4*>(part_o + pr * Dv + 16 * c + 4 * g4) = O[c];
+        return;
+    }
     float oc = 1.f;
     if (sink != nullptr) {
-        const float sk = sink[head];
+        const float sk = sink[head] * 1.4426950408889634f;   // into the base-2 domain of mrow
         const float mn = fmaxf(mrow, sk);
-        oc = mrow == -INFINITY ? 0.f : expf(mrow - mn);
-        lrow = lrow * oc + expf(sk - mn);
+        oc = mrow == -INFINITY ? 0.f : exp2f(mrow - mn);
+        lrow = lrow * oc + exp2f(sk - mn);
     }
     float f = lrow > 0.f ? oc / lrow : 0.f;
     if (gate != nullptr) f *= sigmoidf_(gate[tok * H + head]);
@@ -188,13 +220,42 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
         }
 }
 
+// one wave per (token, head) row: out = sum_z 2^(m_z - m) O_z / (sum_z 2^(m_z - m) l_z + 2^(sink log2 e - m)) * sigmoid(gate)
+__global__ void __launch_bounds__(256) window_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                             const float* __restrict__ sink, const float* __restrict__ gate,
+                                                             uint16_t* __restrict__ out, int64_t rows, int H, int Dv,
+                                                             int nsplit) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    // (the partial maxima are in the base-2 domain: score * scale * log2 e)
+    const float sk = sink != nullptr ? sink[r % H] * 1.4426950408889634f : -INFINITY;
+    float m = sk;
+    for (int z = 0; z < nsplit; ++z) m = fmaxf(m, part_ml[(r * nsplit + z) * 2]);
+    float l = sink != nullptr ? exp2f(sk - m) : 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+        const float mz = part_ml[(r * nsplit + z) * 2];
+        if (mz != -INFINITY) l += exp2f(mz - m) * part_ml[(r * nsplit + z) * 2 + 1];
+    }
+    float f = l > 0.f ? 1.f / l : 0.f;
+    if (gate != nullptr) f *= sigmoidf_(gate[r]);
+    for (int c = lane; c < Dv; c += 64) {
+        float acc = 0.f;
+        for (int z = 0; z < nsplit; ++z) {
+            const float mz = part_ml[(r * nsplit + z) * 2];
+            if (mz != -INFINITY) acc += exp2f(mz - m) * part_o[(r * nsplit + z) * Dv + c];
+        }
+        out[r * Dv + c] = f2bf(acc * f);
+    }
+}
+
 }  // namespace hy
 
 template <int NS, int NCT, int NW>
 static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc, const int32_t* bt,
                            int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
                            const float* gate, uint16_t* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
-                           float scale, int window, int keep, hipStream_t s) {
+                           float scale, int window, int keep, int nsplit, float* part_o, float* part_ml, hipStream_t s) {
     auto kern = hy::window_attention_mfma_kernel<NS, NCT, NW>;
     const int bytes = hy::WKT * (D * 2 + 16) + Dv * (hy::WKT * 2 + 8);
     static int set_bytes = 0;
@@ -202,27 +263,47 @@ static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, con
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         set_bytes = bytes;
     }
-    const dim3 grid(B, (max_q * (H / G) + 16 * NW - 1) / (16 * NW), G);
+    const dim3 grid(B, (max_q * (H / G) + 16 * NW - 1) / (16 * NW) * nsplit, G);
     kern<<<grid, 64 * NW, bytes, s>>>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, H, G, D, Dv, BS, scale,
-                                      window, keep);
+                                      window, keep, nsplit, part_o, part_ml);
 }
 
 bool hy_window_mfma_ok(int ldq, int D, int Dv) { return !(D % 32 || Dv % 16 || D > 256 || Dv > 256 || ldq % 8); }
 
-// false: these sizes are not served here (the caller takes the general kernel).
+// Splits of a row block's key tiles over workgroups (merged by a combine kernel) for launches that would leave most
+// of the chip idle — decode rows, a lone short portion: enough workgroups to cover the CUs twice, at least 2 key
+// tiles per split, at most 16.  The tile count follows from sizes the host knows (the window, or the block table's
+// width when there is none).  1 for float32 and sizes the matrix-core kernel does not serve.
+int hy_window_nsplit(bool f32, int ldq, int B, int max_q, int H, int G, int D, int Dv, int window, int keep, int max_ctx) {
+    if (f32 || !hy_window_mfma_ok(ldq, D, Dv) || B <= 0) return 1;
+    const int rows = max_q * (H / G);
+    const int wgs = B * ((rows + (rows > 64 ? 127 : 63)) / (rows > 64 ? 128 : 64)) * G;
+    if (wgs >= 256) return 1;
+    const int span = window > 0 ? std::min(max_ctx, window + max_q) : max_ctx;
+    const int tiles = span / hy::WKT + 1 + (window > 0 ? (std::min(keep, max_ctx) + hy::WKT - 1) / hy::WKT : 0);
+    int want = (512 + wgs - 1) / wgs;
+    want = std::min(want, std::min(16, tiles / 2));
+    return want < 1 ? 1 : want;
+}
+
+// false: these sizes are not served here (the caller takes the general kernel).  nsplit > 1: part_o float
+// [T * H * nsplit, Dv] and part_ml float [T * H * nsplit, 2] scratch.
 bool launch_hy_window_attention_mfma(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc,
                                      const int32_t* bt, int max_blocks, const int32_t* q_start, const int32_t* pos,
                                      const float* sink, const float* gate, uint16_t* out, int B, int max_q, int H, int G,
-                                     int D, int Dv, int BS, float scale, int window, int keep, hipStream_t s) {
+                                     int D, int Dv, int BS, float scale, int window, int keep, int nsplit, float* part_o,
+                                     float* part_ml, int64_t total_rows, hipStream_t s) {
     if (!hy_window_mfma_ok(ldq, D, Dv)) return false;
     if (B == 0 || max_q == 0) return true;
-#define HY_WAM(NS, NCT, NW) wa_mfma_launch<NS, NCT, NW>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, B, max_q, H, G, D, Dv, BS, scale, window, keep, s)
+#define HY_WAM(NS, NCT, NW) wa_mfma_launch<NS, NCT, NW>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, B, max_q, H, G, D, Dv, BS, scale, window, keep, nsplit, part_o, part_ml, s)
     // 8 waves per workgroup when a sequence brings more than 64 rows per key/value head: a staged tile then serves
     // 128 rows and every SIMD holds two waves
     const bool nw8 = max_q * (H / G) > 64;
     if (D <= 128 && Dv <= 128) { if (nw8) HY_WAM(4, 8, 8); else HY_WAM(4, 8, 4); }
     else { if (nw8) HY_WAM(8, 16, 8); else HY_WAM(8, 16, 4); }
 #undef HY_WAM
+    if (nsplit > 1)
+        hy::window_combine_kernel<<<(unsigned)((total_rows + 3) / 4), 256, 0, s>>>(part_o, part_ml, sink, gate, out, total_rows, H, Dv, nsplit);
     return true;
 }
 
