@@ -271,17 +271,17 @@ static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, con
 bool hy_window_mfma_ok(int ldq, int D, int Dv) { return !(D % 32 || Dv % 16 || D > 256 || Dv > 256 || ldq % 8); }
 
 // Splits of a row block's key tiles over workgroups (merged by a combine kernel) for launches that would leave most
-// of the chip idle — decode rows, a lone short portion: enough workgroups to cover the CUs twice, at least 2 key
+// of the chip idle — decode rows, a lone short portion: enough workgroups to cover the CUs four times, at least 2 key
 // tiles per split, at most 16.  The tile count follows from sizes the host knows (the window, or the block table's
 // width when there is none).  1 for float32 and sizes the matrix-core kernel does not serve.
 int hy_window_nsplit(bool f32, int ldq, int B, int max_q, int H, int G, int D, int Dv, int window, int keep, int max_ctx) {
     if (f32 || !hy_window_mfma_ok(ldq, D, Dv) || B <= 0) return 1;
     const int rows = max_q * (H / G);
     const int wgs = B * ((rows + (rows > 64 ? 127 : 63)) / (rows > 64 ? 128 : 64)) * G;
-    if (wgs >= 256) return 1;
+    if (wgs >= 512) return 1;
     const int span = window > 0 ? std::min(max_ctx, window + max_q) : max_ctx;
     const int tiles = span / hy::WKT + 1 + (window > 0 ? (std::min(keep, max_ctx) + hy::WKT - 1) / hy::WKT : 0);
-    int want = (512 + wgs - 1) / wgs;
+    int want = (1024 + wgs - 1) / wgs;
     want = std::min(want, std::min(16, tiles / 2));
     return want < 1 ? 1 : want;
 }
