@@ -181,39 +181,42 @@ def test_rotation_frequencies_follow_the_wavelength_rule():
 
 
 # ---- the visible set of the windowed attention, key by key --------------------------------------------------------
-@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("device,dt", [("cpu", torch.float32), pytest.param("cuda", torch.float32, marks=pytest.mark.gpu),
+                                       pytest.param("cuda", torch.bfloat16, marks=pytest.mark.gpu)])
 @pytest.mark.parametrize("window,keep", [(9, 3), (16, 0), (64, 17), (70, 70), (1, 1), (0, 0), (130, 2)])
-def test_window_visible_set(device, window, keep):
+def test_window_visible_set(device, dt, window, keep):
     """Zero queries make every visible key weigh the same, and one-hot values make the output of a query its
     visibility pattern: out[i, j] = 1 / (visible(i) + exp(sink)) for the keys j that i sees, else 0.  Prompt portions
-    that start and end anywhere beside decode rows, pages dealt out of order."""
+    that start and end anywhere beside decode rows, pages dealt out of order.  (bfloat16 at these sizes runs the
+    matrix-core kernel, with the key tiles of its few-row launches split over workgroups.)"""
     from chronos.ops import hybrid as hops
 
-    dt = torch.float32
-    ctx, bs, H, G, D = 200, 16, 2, 1, 8
+    ctx, bs, H, G, D = 192, 16, 2, 1, 32
     nb = ctx // bs + 2
-    kc = torch.randn(nb, bs, G, D, dtype=dt)
+    kc = torch.randn(nb, bs, G, D).to(dt)
     vc = torch.zeros(nb, bs, G, ctx, dtype=dt)
     pages = list(range(nb - 1, 0, -1))
     for j in range(ctx):
         vc[pages[j // bs], j % bs, 0, j] = 1.0
     sink = torch.tensor([0.3, -1.0])
-    for lo, hi in [(0, 200), (0, 1), (63, 65), (64, 130), (127, 200), (199, 200), (5, 6), (150, 151)]:
+    tol = 1e-6 if dt == torch.float32 else 4e-3
+    for lo, hi in [(0, 192), (0, 1), (63, 65), (64, 130), (127, 192), (191, 192), (5, 6), (150, 151)]:
         n = hi - lo
-        qkv = torch.zeros(n, H * D, dtype=dt)
+        qkv = torch.zeros(n, (H + G) * D + G * ctx, dtype=dt)
         i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=device)  # noqa: E731
         bt = torch.zeros(2, nb, dtype=torch.int32)
         bt[1, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
         # (sequence 0 of the batch brings nothing; the portion belongs to sequence 1)
         out = hops.window_attention(qkv.to(device), kc.to(device), vc.to(device), bt.to(device), i32([0, 0, n]),
                                     i32(list(range(lo, hi))), sink.to(device), None, 1.0, window, keep, H, dt, n)
-        out = out.view(n, H, ctx).cpu()
+        out = out.view(n, H, ctx).float().cpu()
         for r, i in enumerate(range(lo, hi)):
             vis = torch.tensor([1.0 if plain.visible(i, j, dict(size=window, keep_first=keep) if window else None) else 0.0
                                 for j in range(ctx)])
             for h in range(H):
                 want = vis / (vis.sum() + torch.exp(sink[h]))
-                assert float((out[r, h] - want).abs().max()) < 1e-6, (lo, hi, i, h)
+                assert torch.equal(out[r, h] != 0, vis != 0), (lo, hi, i, h)
+                assert float((out[r, h] - want).abs().max()) <= tol * float(want.max()) + 1e-7, (lo, hi, i, h)
 
 
 @pytest.mark.parametrize("device", DEVICES)
