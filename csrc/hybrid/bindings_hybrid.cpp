@@ -55,7 +55,7 @@ void launch_hy_delta_prep(const void*, int, const float*, const float*, float*, 
                           float, bool, hipStream_t);
 bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const float*, float, const float*, bool,
                            const float*, const int32_t*, const int32_t*, const int32_t*, float*, float*, int, int, int, int,
-                           int, bool, hipStream_t);
+                           int, int, bool, hipStream_t);
 void launch_hy_moe_route_topk(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
                               hipStream_t);
 void launch_hy_moe_glu_grouped(const uint16_t*, const int32_t*, const float*, const uint16_t*, const uint16_t*, uint16_t*,
@@ -470,7 +470,7 @@ Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t 
         proj.data_ptr(), (int)C, (int)q_off, (int)k_off, (int)v_off, qscale ? qscale->data_ptr<float>() : nullptr,
         kscale ? kscale->data_ptr<float>() : nullptr, (float)q_mul, decay.data_ptr<float>(), chd,
         beta ? beta->data_ptr<float>() : nullptr, q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(),
-        slots.data_ptr<int32_t>(), S.data_ptr<float>(), o.data_ptr<float>(), (int)B, (int)HK, (int)H, (int)D, (int)Dv,
+        slots.data_ptr<int32_t>(), S.data_ptr<float>(), o.data_ptr<float>(), (int)T, (int)B, (int)HK, (int)H, (int)D, (int)Dv,
         f32(proj), stream());
     TORCH_CHECK(ok, "chronos hybrid op: linear_scan keeps a state column in registers, D <= 256 (got ", D, ")");
     return o;

@@ -100,36 +100,42 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(const T* __restrict__ y
 }
 
 constexpr int kScanTC = 16;  // tokens per LDS stage
-constexpr int kScanRG = 4;   // row groups per wave: lane = 16 columns x 4 groups of DP / 4 state rows
-constexpr int kScanCW = 64 / kScanRG;
+// row groups per wave: a lane holds DP / RG rows of one of the wave's 64 / RG columns.  4 for decode rows (16
+// columns = 64-byte runs of the state per row), 8 for prompt portions (half the per-token chain per wave, twice the
+// waves)
+constexpr int kScanRGDecode = 4, kScanRGPrefill = 8;
 
 template <typename T> __device__ __forceinline__ T zero_of();
 template <> __device__ __forceinline__ float zero_of<float>() { return 0.f; }
 template <> __device__ __forceinline__ uint16_t zero_of<uint16_t>() { return 0; }
 
-// 256 threads: wave w owns value columns 16 w .. 16 w + 15 of the workgroup's 64; a lane holds DP / 4 rows of one
+// 256 threads: wave w owns 64 / RG value columns of the workgroup's 4 x 64 / RG; a lane holds DP / RG rows of one
 // column.  LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64] | per token: decay, beta,
 // q scale, k scale.  The next stage's global loads are issued before the current stage's tokens are processed and
 // land in LDS afterwards, so the token loop never waits on global memory; the scales of q and k are folded into
 // per-token scalars (S^T k_hat = s_k S^T k, k_hat u^T = k (s_k u)^T, S^T q_hat = s_q S^T q).
-template <typename T, int DP, bool DELTA, bool CHD>
+// PIPE: the one-pass token loops with LDS rows prefetched (more registers: for launches with prompt portions);
+// without it the plain order of operations, whose lower register count suits launches of single decode rows, which
+// are bound by the state's bytes.
+template <typename T, int DP, bool DELTA, bool CHD, bool PIPE>
 __global__ void __launch_bounds__(256) linear_scan_kernel(
         const T* __restrict__ proj, int ldp, int q_off, int k_off, int v_off, const float* __restrict__ qscale,
         const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, const float* __restrict__ beta,
         const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots,
         float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv) {
-    constexpr int TC = kScanTC, RG = kScanRG, CW = kScanCW, RL = DP / RG, NE = TC * DP / 256;
+    constexpr int TC = kScanTC, RG = PIPE ? kScanRGPrefill : kScanRGDecode, CW = 64 / RG, RL = DP / RG;
+    constexpr int NE = TC * DP / 256, WC = 4 * CW;  // WC: value columns of the workgroup
     __shared__ __attribute__((aligned(16))) float qs[TC * DP];
     __shared__ __attribute__((aligned(16))) float ks[TC * DP];
     __shared__ __attribute__((aligned(16))) float ds[CHD ? TC * DP : 4];
-    __shared__ float vs[TC * 64];
+    __shared__ float vs[TC * WC];
     __shared__ float gs[TC], bs[TC], qsc[TC], ksc[TC];
     const int b = blockIdx.x, hd = blockIdx.y;
     const int t0 = q_start[b], t1 = q_start[b + 1];
     if (t1 <= t0) return;
     const int hk = hd / (H / HK);
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, rg = lane / CW, c = lane % CW;
-    const int col0 = blockIdx.z * 64;
+    const int col0 = blockIdx.z * WC;
     const int col = col0 + wv * CW + c;
     const bool live = col < Dv;
     float* Sp = S + (((int64_t)slots[b] * H + hd) * D) * Dv + col;
@@ -142,7 +148,8 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         for (int i = 0; i < RL; ++i) st_[i] = 0.f;
     }
     // staging registers of one stage: element e of thread x is (token e' = (x + 256 e) / DP, row (x + 256 e) % DP)
-    T qraw[NE], kraw[NE], vraw[4];
+    constexpr int NV = (TC * WC + 255) / 256;
+    T qraw[NE], kraw[NE], vraw[NV];
     float draw[CHD ? NE : 1], sraw[4];
     auto fetch = [&](int tb) {
         const int nt = min(TC, t1 - tb);
@@ -156,8 +163,8 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
             if constexpr (CHD) draw[e] = ok ? decay[(t * H + hd) * D + r] : 0.f;
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int i = threadIdx.x + 256 * e, tt = i >> 6, cc = col0 + (i & 63);
+        for (int e = 0; e < NV; ++e) {
+            const int i = threadIdx.x + 256 * e, tt = i / WC, cc = col0 + i % WC;
             vraw[e] = (tt < nt && cc < Dv) ? proj[(int64_t)(tb + tt) * ldp + v_off + hd * Dv + cc] : zero_of<T>();
         }
         if (threadIdx.x < TC) {
@@ -178,7 +185,8 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
             if constexpr (CHD) ds[i] = draw[e];
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) vs[threadIdx.x + 256 * e] = ld<T>(&vraw[e]);
+        for (int e = 0; e < NV; ++e)
+            if (threadIdx.x + 256 * e < TC * WC) vs[threadIdx.x + 256 * e] = ld<T>(&vraw[e]);
         if (threadIdx.x < TC) {
             gs[threadIdx.x] = sraw[0];
             bs[threadIdx.x] = sraw[1];
@@ -193,49 +201,121 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         land();
         __syncthreads();
         if (tb + TC < t1) fetch(tb + TC);
-        for (int tt = 0; tt < nt; ++tt) {
-            const f32x4* q4 = reinterpret_cast<const f32x4*>(qs + tt * DP + rg * RL);
-            const f32x4* k4 = reinterpret_cast<const f32x4*>(ks + tt * DP + rg * RL);
-            float g = 1.f;
-            if constexpr (CHD) {
-                const f32x4* d4 = reinterpret_cast<const f32x4*>(ds + tt * DP + rg * RL);
+        // a lane's RL rows of token tt's staged row, as registers (one batch of 16-byte LDS reads)
+        auto ldrow = [&](const float* base, int tt, float (&dst)[RL]) {
+            const f32x4* p4 = reinterpret_cast<const f32x4*>(base + tt * DP + rg * RL);
 #pragma unroll
-                for (int i = 0; i < RL; i += 4) {
-                    const f32x4 dv = d4[i >> 2];
-                    st_[i] *= dv[0]; st_[i + 1] *= dv[1]; st_[i + 2] *= dv[2]; st_[i + 3] *= dv[3];
-                }
-            } else {
-                g = gs[tt];
+            for (int i = 0; i < RL; i += 4) {
+                const f32x4 v = p4[i >> 2];
+                dst[i] = v[0]; dst[i + 1] = v[1]; dst[i + 2] = v[2]; dst[i + 3] = v[3];
             }
-            const float sk = ksc[tt];
-            float u = vs[tt * 64 + wv * CW + c];
-            if constexpr (DELTA) {
+        };
+        auto rsum = [&](float x) {   // over the row groups
+#pragma unroll
+            for (int o = CW; o < 64; o <<= 1) x += __shfl_xor(x, o, 64);
+            return x;
+        };
+        if constexpr (PIPE && DELTA && !CHD) {
+            // The delta rule with one decay per head, one pass over the state per token: the pass that writes token
+            // t and reads it out also forms S^T k of token t + 1 (its decay is a scalar factor applied afterwards),
+            // so the two cross-lane sums of a token run side by side and the next token's k rows are read from LDS
+            // while the current token is computed.  Two register sets of k rows alternate.
+            float ka[RL], kb[RL], qc[RL];
+            ldrow(ks, 0, ka);
+            float p;
+            {
                 float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
                 for (int i = 0; i < RL; i += 4) {
-                    const f32x4 kv = k4[i >> 2];
-                    p0 += st_[i] * kv[0]; p1 += st_[i + 1] * kv[1]; p2 += st_[i + 2] * kv[2]; p3 += st_[i + 3] * kv[3];
+                    p0 += st_[i] * ka[i]; p1 += st_[i + 1] * ka[i + 1]; p2 += st_[i + 2] * ka[i + 2]; p3 += st_[i + 3] * ka[i + 3];
                 }
-                float p = (p0 + p1) + (p2 + p3);
-                p += __shfl_xor(p, 16, 64);
-                p += __shfl_xor(p, 32, 64);
-                u = bs[tt] * (u - g * sk * p);
+                p = rsum((p0 + p1) + (p2 + p3));
             }
-            const float uk = u * sk;
-            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+            auto step = [&](int tt, float (&kc)[RL], float (&kn)[RL]) {
+                ldrow(qs, tt, qc);
+                if (tt + 1 < nt) ldrow(ks, tt + 1, kn);   // (else kn keeps old rows: the sum below is not used)
+                const float g = gs[tt], sk = ksc[tt];
+                const float u = bs[tt] * (vs[tt * WC + wv * CW + c] - g * sk * p);
+                const float uk = u * sk;
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f, n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;
 #pragma unroll
-            for (int i = 0; i < RL; i += 4) {
-                const f32x4 kv = k4[i >> 2], qv = q4[i >> 2];
-                st_[i] = g * st_[i] + kv[0] * uk;
-                st_[i + 1] = g * st_[i + 1] + kv[1] * uk;
-                st_[i + 2] = g * st_[i + 2] + kv[2] * uk;
-                st_[i + 3] = g * st_[i + 3] + kv[3] * uk;
-                a0 += st_[i] * qv[0]; a1 += st_[i + 1] * qv[1]; a2 += st_[i + 2] * qv[2]; a3 += st_[i + 3] * qv[3];
+                for (int i = 0; i < RL; i += 4) {
+                    st_[i] = g * st_[i] + kc[i] * uk;
+                    st_[i + 1] = g * st_[i + 1] + kc[i + 1] * uk;
+                    st_[i + 2] = g * st_[i + 2] + kc[i + 2] * uk;
+                    st_[i + 3] = g * st_[i + 3] + kc[i + 3] * uk;
+                    a0 += st_[i] * qc[i]; a1 += st_[i + 1] * qc[i + 1]; a2 += st_[i + 2] * qc[i + 2]; a3 += st_[i + 3] * qc[i + 3];
+                    n0 += st_[i] * kn[i]; n1 += st_[i + 1] * kn[i + 1]; n2 += st_[i + 2] * kn[i + 2]; n3 += st_[i + 3] * kn[i + 3];
+                }
+                const float a = rsum((a0 + a1) + (a2 + a3));
+                p = rsum((n0 + n1) + (n2 + n3));
+                if (live && rg == 0) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = a * qsc[tt];
+            };
+            for (int tt = 0; tt < nt; tt += 2) {
+                step(tt, ka, kb);
+                if (tt + 1 < nt) step(tt + 1, kb, ka);
             }
-            float a = (a0 + a1) + (a2 + a3);
-            a += __shfl_xor(a, 16, 64);
-            a += __shfl_xor(a, 32, 64);
-            if (live && rg == 0) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = a * qsc[tt];
+        } else if constexpr (PIPE && !DELTA && CHD) {
+            // Per-row decays without the delta correction (gated linear attention): one fused pass per token,
+            // S <- d S + k v^T and o = S^T q; the next token's rows are read from LDS during the current pass.
+            float da[RL], ka[RL], qa[RL], db[RL], kb[RL], qb[RL];
+            ldrow(ds, 0, da); ldrow(ks, 0, ka); ldrow(qs, 0, qa);
+            auto step = [&](int tt, float (&dc)[RL], float (&kc)[RL], float (&qc)[RL], float (&dn)[RL], float (&kn)[RL], float (&qn)[RL]) {
+                if (tt + 1 < nt) { ldrow(ds, tt + 1, dn); ldrow(ks, tt + 1, kn); ldrow(qs, tt + 1, qn); }
+                const float uk = vs[tt * WC + wv * CW + c] * ksc[tt];
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+                for (int i = 0; i < RL; i += 4) {
+                    st_[i] = dc[i] * st_[i] + kc[i] * uk;
+                    st_[i + 1] = dc[i + 1] * st_[i + 1] + kc[i + 1] * uk;
+                    st_[i + 2] = dc[i + 2] * st_[i + 2] + kc[i + 2] * uk;
+                    st_[i + 3] = dc[i + 3] * st_[i + 3] + kc[i + 3] * uk;
+                    a0 += st_[i] * qc[i]; a1 += st_[i + 1] * qc[i + 1]; a2 += st_[i + 2] * qc[i + 2]; a3 += st_[i + 3] * qc[i + 3];
+                }
+                const float a = rsum((a0 + a1) + (a2 + a3));
+                if (live && rg == 0) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = a * qsc[tt];
+            };
+            for (int tt = 0; tt < nt; tt += 2) {
+                step(tt, da, ka, qa, db, kb, qb);
+                if (tt + 1 < nt) step(tt + 1, db, kb, qb, da, ka, qa);
+            }
+        } else {
+            // the plain order of operations
+            for (int tt = 0; tt < nt; ++tt) {
+                float kc[RL], qc[RL];
+                ldrow(ks, tt, kc); ldrow(qs, tt, qc);
+                float g = 1.f;
+                if constexpr (CHD) {
+                    float dc[RL];
+                    ldrow(ds, tt, dc);
+#pragma unroll
+                    for (int i = 0; i < RL; ++i) st_[i] *= dc[i];
+                } else {
+                    g = gs[tt];
+                }
+                const float sk = ksc[tt];
+                float u = vs[tt * WC + wv * CW + c];
+                if constexpr (DELTA) {
+                    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+#pragma unroll
+                    for (int i = 0; i < RL; i += 4) {
+                        p0 += st_[i] * kc[i]; p1 += st_[i + 1] * kc[i + 1]; p2 += st_[i + 2] * kc[i + 2]; p3 += st_[i + 3] * kc[i + 3];
+                    }
+                    u = bs[tt] * (u - g * sk * rsum((p0 + p1) + (p2 + p3)));
+                }
+                const float uk = u * sk;
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+                for (int i = 0; i < RL; i += 4) {
+                    st_[i] = g * st_[i] + kc[i] * uk;
+                    st_[i + 1] = g * st_[i + 1] + kc[i + 1] * uk;
+                    st_[i + 2] = g * st_[i + 2] + kc[i + 2] * uk;
+                    st_[i + 3] = g * st_[i + 3] + kc[i + 3] * uk;
+                    a0 += st_[i] * qc[i]; a1 += st_[i + 1] * qc[i + 1]; a2 += st_[i + 2] * qc[i + 2]; a3 += st_[i + 3] * qc[i + 3];
+                }
+                const float a = rsum((a0 + a1) + (a2 + a3));
+                if (live && rg == 0) o[((int64_t)(tb + tt) * H + hd) * Dv + col] = a * qsc[tt];
+            }
         }
     }
     if (live) {
@@ -269,22 +349,31 @@ void launch_hy_delta_prep(const void* y, int ldy, const float* ab, const float* 
 }
 
 template <typename T, int DP, bool DELTA, bool CHD>
-static void linear_scan_launch(const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
+static void linear_scan_launch(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                                const float* kscale, float q_mul, const float* decay, const float* beta,
                                const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
                                int HK, int H, int D, int Dv, hipStream_t s) {
-    const dim3 grid(B, H, (Dv + 63) / 64);
-    hy::linear_scan_kernel<T, DP, DELTA, CHD><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
-                                                                  beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
+    constexpr bool HAS_PIPE = DELTA != CHD;   // the two combinations with a pipelined token loop
+    if constexpr (HAS_PIPE) {
+        if (pipe) {
+            const dim3 grid(B, H, (Dv + 4 * (64 / hy::kScanRGPrefill) - 1) / (4 * (64 / hy::kScanRGPrefill)));
+            hy::linear_scan_kernel<T, DP, DELTA, CHD, true><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
+                                                                                beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
+            return;
+        }
+    }
+    const dim3 grid(B, H, (Dv + 4 * (64 / hy::kScanRGDecode) - 1) / (4 * (64 / hy::kScanRGDecode)));
+    hy::linear_scan_kernel<T, DP, DELTA, CHD, false><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
+                                                                         beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
 }
 
 template <typename T, bool DELTA, bool CHD>
-static bool linear_scan_d(const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
+static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                           const float* kscale, float q_mul, const float* decay, const float* beta, const int32_t* q_start,
                           const int32_t* pos0, const int32_t* slots, float* S, float* o, int B, int HK, int H, int D,
                           int Dv, hipStream_t s) {
 #define HY_LS(DP)                                                                                                     \
-    linear_scan_launch<T, DP, DELTA, CHD>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, \
+    linear_scan_launch<T, DP, DELTA, CHD>(pipe, proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, \
                                           pos0, slots, S, o, B, HK, H, D, Dv, s)
     if (D <= 32) HY_LS(32);
     else if (D <= 64) HY_LS(64);
@@ -299,12 +388,13 @@ static bool linear_scan_d(const T* proj, int ldp, int q_off, int k_off, int v_of
 // Returns false when D has no instantiation (D > 256).
 bool launch_hy_linear_scan(const void* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                            const float* kscale, float q_mul, const float* decay, bool chd, const float* beta,
-                           const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
-                           int HK, int H, int D, int Dv, bool f32, hipStream_t s) {
+                           const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int T,
+                           int B, int HK, int H, int D, int Dv, bool f32, hipStream_t s) {
     if (B == 0) return true;
+    const bool pipe = T > B;   // some sequence brings more than one token
     const bool delta = beta != nullptr;
 #define HY_LSD(T, DELTA, CHD)                                                                                        \
-    return linear_scan_d<T, DELTA, CHD>((const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, \
+    return linear_scan_d<T, DELTA, CHD>(pipe, (const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, \
                                         q_start, pos0, slots, S, o, B, HK, H, D, Dv, s)
     if (f32) {
         if (delta && chd) HY_LSD(float, true, true);
