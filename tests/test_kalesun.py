@@ -362,6 +362,72 @@ def test_router_weights_are_the_softmax_over_the_chosen(device):
     assert sorted(idx[0].tolist()) == [1, 4] and torch.allclose(wt.sum(-1).cpu(), torch.ones(6))
 
 
+# ---- designs drawn at random: sizes, order of layers, windows, constants ---------------------------------------------
+def _random_design(seed, tile_sizes=False):
+    """A configuration drawn at random.  ``tile_sizes``: head sizes and widths on the grids of the matrix-core
+    kernels (attention dim % 32, vdim % 16; experts and width on the 128 grid), so that bfloat16 runs take them."""
+    import random
+
+    r = random.Random(seed)
+    pick = r.choice
+    layers = []
+    kv, vd = pick([1, 2, 3]), pick([16, 48, 80]) if tile_sizes else pick([6, 20, 34])
+    for _ in range(r.randint(3, 6)):
+        kind = pick("adg")
+        if kind == "a":
+            dim = pick([32, 64, 96]) if tile_sizes else pick([6, 10, 24])
+            dims = pick([0, dim, dim // 2 // 2 * 2, 2])
+            mixer = _attn(heads=kv * pick([1, 2, 4]), kv_heads=kv, dim=dim, vdim=vd, scale=pick([0.1, 0.5, 1.5]),
+                          size=pick([0, 1, 5, 16, 33, 64, 100]), keep=pick([0, 1, 7, 30]), dims=dims,
+                          base=pick([100.0, 1e4, 5e5]), scaling=pick([True, False]), v_mix=pick([True, True, False]))
+        elif kind == "d":
+            hk = pick([1, 2])
+            mixer = _delta(heads=hk * pick([1, 2, 3]), kv_heads=hk, dim=pick([4, 12, 32, 40]), vdim=pick([8, 24, 72]),
+                           conv=pick([1, 2, 3, 4, 6]))
+        else:
+            mixer = _gla(heads=pick([1, 2, 5]), dim=pick([4, 12, 32]), vdim=pick([8, 24, 72]), tau=pick([1.0, 4.0, 16.0]),
+                         rank=pick([1, 3, 8]))
+        f = pick(["dense", "moe", "moe", None])
+        ff = 128 if tile_sizes else pick([8, 24, 40])
+        if f == "dense":
+            mlp = _dense(ff, pick([0.5, 1.0, 7.0]))
+        elif f == "moe":
+            e = pick([1, 2, 5, 9])
+            mlp = _moe(e, r.randint(1, e), ff, pick([0.5, 1.5, 7.0]))
+        else:
+            mlp = None
+        layers.append((mixer, mlp))
+    return _config(layers, width=128 if tile_sizes else pick([24, 40, 72]), vocab=pick([50, 131, 300]),
+                   alpha=pick([1.0, 2.0, 0.7]), eps=pick([1e-6, 1e-5]))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5])
+def test_designs_drawn_at_random(device, seed):
+    cfg = _random_design(seed)
+    eng, tensors = _engine(cfg, device, slots=3, max_len=160, blocks=14)
+    reqs = _requests(cfg, [90, 37, 2, 61], seed=seed)
+    sched = [[("r0", 40), ("r1", 2)], [("r0", 1), ("r1", 33), ("r2", 2)], [("r0", 2), ("r1", 1)], [("r0", 30), ("r1", 1), ("r3", 17)],
+             [("r0", 1), ("r3", 3)]] + [[("r0", 1), ("r3", 1)] for _ in range(16)] + [[("r3", 25)]]
+    _check(eng, tensors, cfg, sched, reqs, "fp32")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_designs_drawn_at_random_on_the_matrix_cores(seed):
+    """bfloat16 at sizes the matrix-core attention and the grouped experts serve, against the oracle; and the same
+    requests cut differently must agree with each other far more closely than bfloat16 rounding."""
+    cfg = _random_design(seed, tile_sizes=True)
+    eng, tensors = _engine(cfg, "cuda", "bf16", slots=3, max_len=160, blocks=14)
+    reqs = _requests(cfg, [90, 61], seed=seed)
+    a = _replay(eng, [[("r0", 90)], [("r1", 61)]], reqs)
+    b = _replay(eng, [[("r0", 40), ("r1", 2)], [("r0", 1), ("r1", 33)], [("r0", 30), ("r1", 25)], [("r0", 19), ("r1", 1)]], reqs)
+    for name, toks in reqs.items():
+        want = _want(cfg, tensors, toks)
+        assert not _bad(a[name].cpu(), want, "bf16"), (name, _errs(a[name].cpu(), want))
+        assert not _bad(b[name].cpu(), want, "bf16"), (name, _errs(b[name].cpu(), want))
+
+
 # ---- generation through the engine's own entry point and scheduler ------------------------------------------------
 def _greedy(cfg, tensors, prompt, n):
     m = plain.Plain(cfg, tensors)
