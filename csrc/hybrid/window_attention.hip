@@ -7,7 +7,8 @@
 //                     the token's page and slot of kc [NB, BS, G, D] / vc [NB, BS, G, Dv].
 //   window_attention  the general kernel (vector ALUs, float or bfloat16, any sizes): a workgroup takes one sequence,
 //                     one key/value head and up to 16 consecutive query tokens with all the query heads of that
-//                     group (at most 64 (token, head) rows); 64-key tiles of the cache are staged in LDS; lanes are keys for the scores (float
+//                     group (at most 64 (token, head) rows, fewer when the LDS asks for it); 64-key tiles of the
+//                     cache are staged in LDS; lanes are keys for the scores (float
 //                     accumulation, online softmax in float) and value columns for the output.  The key range of a
 //                     tile of queries is [0, keep_first) and [first query - window + 1, last query]; tiles of keys
 //                     between the two are never touched, and each row masks by its own position:

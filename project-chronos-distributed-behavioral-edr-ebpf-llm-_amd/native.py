@@ -6,8 +6,8 @@ to the GPU box and show up as in-tree loads):
   _sensor_native   g++      csrc/sensor_host/*.cpp      shared eBPF filter policy, data_t codec, chain tracker
   _constrain_native g++     csrc/constrain/*.cpp        JSON / verdict-schema token automaton compiler, tokenizer trie
   _C               hipcc    csrc/kernels/*.hip          gfx950 HIP kernels (MFMA/LDS) as torch ops
-  _H               hipcc    csrc/hybrid/*.hip           the hybrid-decoder kernels (recurrent state, latent attention,
-                                                        mixture of experts) as torch ops, loadable without _C
+  _H               hipcc    csrc/hybrid/*.hip           the hybrid-decoder kernels (recurrent state, latent and windowed
+                                                        attention, mixture of experts) as torch ops, loadable without _C
 
 The HIP library is compiled with hipcc directly (``--offload-arch=gfx950``), not through torch's cpp_extension, so no
 hipify pass ever touches the sources.  Rebuilds are keyed on a hash of sources + flags.

@@ -1,6 +1,6 @@
-"""Ops of the hybrid decoders (recurrent matrix-memory layers, latent attention, mixtures of experts, layer norms on
-a float32 residual stream): gfx950 HIP kernels on the GPU (csrc/hybrid/*.hip), the PyTorch references of
-:mod:`.hybrid_ref` on the CPU.
+"""Ops of the hybrid decoders (recurrent matrix-memory layers, linear-state recurrences, latent and windowed
+attention, mixtures of experts, layer and RMS norms on a float32 residual stream): gfx950 HIP kernels on the GPU
+(csrc/hybrid/*.hip), the PyTorch references of :mod:`.hybrid_ref` on the CPU.
 
 As everywhere in :mod:`chronos.ops` a GPU tensor never falls back silently: it goes to ``torch.ops.chronos.hy_*`` or
 raises.  ``CHRONOS_HYBRID_REF=1`` is a bring-up switch that runs the PyTorch references on GPU tensors (it syncs with
